@@ -15,7 +15,7 @@ int r32_xielu(const void*, int, const void*, void*, int, int, int, int, hipStrea
 int r32_residual_add_scaled(float*, const void*, float, long long, int, hipStream_t);
 int r32_residual_add_partials(float*, const float*, int, float, long long, hipStream_t);
 int r32_window_attn(const float*, const void*, const void*, long long, long long, int, const int*, const int*, int,
-                    const int*, int, const float*, const float*, int, void*, int, int, int, int, int, int, int,
+                    const int*, int, const float*, const float*, const float*, int, void*, int, int, int, int, int, int, int,
                     hipStream_t);
 int r32_window_attn_mfma_ok(int, int);
 int r32_window_attn_mfma(const float*, const void*, const void*, long long, long long, int, const int*, const int*,
@@ -42,10 +42,23 @@ int r32_rmsnorm_rows(const float*, const long long*, const float*, void*, int, i
 int r32_gelu_mul_rows(const void*, int, const void*, int, int, const int*, int, void*, int, int, int, hipStream_t);
 int r32_stack_mix(const float*, long long, const float*, int, float*, long long, hipStream_t);
 int r32_router_max_outputs();
-int r32_router(const float*, const float*, int, int, int, int, int*, float*, int*, int*, int*, int*, int*, int*, hipStream_t);
+int r32_router(const float*, const float*, const float*, int, int, int, int, int, int*, float*, int*, int*, int*, int*, int*,
+               int*, hipStream_t);
 int r32_expert_rows(const void*, int, const int*, const int*, const int*, int, const void*, const void*, float*, int, int,
                     int, int, hipStream_t);
-int r32_moe_combine(const void*, int, const int*, const float*, const void*, int, int, int, float*, int, int, hipStream_t);
+int r32_moe_combine(const void*, int, const int*, const float*, const void*, int, int, int, float*, int, const void*, int, int,
+                    hipStream_t);
+int r32_latent_kv_write(const void*, int, int, int, int, const float*, const float*, const float*, float, const int*,
+                        const int*, void*, int, void*, void*, long long, long long, int, int, int, float, int, int,
+                        hipStream_t);
+int r32_latent_q_rows(const void*, int, int, int, const float*, int, const float*, float, float, const int*, float*, int, int,
+                      int, int, hipStream_t);
+int r32_retention_max_dim();
+int r32_retention_prep(const void*, int, int, const float*, float, const int*, float*, int, int, int, int, float, int,
+                       hipStream_t);
+int r32_retention(const float*, const void*, int, const float*, float*, long long, const int*, const int*, const int*, float*,
+                  int, int, int, int, int, int, hipStream_t);
+int r32_glu(const void*, int, void*, int, int, int, int, float, float, int, hipStream_t);
 }
 
 namespace {
@@ -184,8 +197,10 @@ void residual_add_partials(Tensor x, Tensor parts, double m) {
 
 // q fp32 [T, H*D]; out [T, >= H*Dv] row-dense view of the cache dtype; block_tables [items, width] int32;
 // cu_q: int32 [items + 1] for prompt portions, absent when row t is item t.
+// sink: fp32 [H], exp(sink_h) joins head h's softmax denominator (no key, no value), or absent.
 void window_attn(Tensor q, Tensor k_cache, Tensor v_cache, Tensor positions, c10::optional<Tensor> cu_q,
-                 Tensor block_tables, Tensor r1, Tensor r2, int64_t window, Tensor out, int64_t H, int64_t G) {
+                 Tensor block_tables, Tensor r1, Tensor r2, int64_t window, Tensor out, int64_t H, int64_t G,
+                 c10::optional<Tensor> sink) {
   want(q, torch::kFloat32, "window_attn q");
   const int f = act_f32(k_cache, "window_attn k_cache");
   want(positions, torch::kInt32, "window_attn positions");
@@ -211,9 +226,15 @@ void window_attn(Tensor q, Tensor k_cache, Tensor v_cache, Tensor positions, c10
   } else {
     TORCH_CHECK(items >= T, "window_attn: one table row per query row");
   }
+  const float* sk = nullptr;
+  if (sink.has_value()) {
+    want(*sink, torch::kFloat32, "window_attn sink");
+    TORCH_CHECK(sink->numel() == H, "window_attn: sink [H]");
+    sk = sink->data_ptr<float>();
+  }
   done(r32_window_attn(q.data_ptr<float>(), k_cache.data_ptr(), v_cache.data_ptr(), (long long)k_cache.stride(0),
                        (long long)v_cache.stride(0), BS, positions.data_ptr<int>(), cu, items, block_tables.data_ptr<int>(),
-                       width, r1.data_ptr<float>(), r2.data_ptr<float>(), (int)window, out.data_ptr(), ldo, T, (int)H, (int)G,
+                       width, r1.data_ptr<float>(), r2.data_ptr<float>(), sk, (int)window, out.data_ptr(), ldo, T, (int)H, (int)G,
                        D, Dv, f, stream()), "window_attn");
 }
 
@@ -529,10 +550,14 @@ int64_t router_max_outputs() { return r32_router_max_outputs(); }
 
 // z fp32 [T, NE] router logits, corr fp32 [NE]; the first E outputs are real experts.  Returns
 // (ids [T,k] i32, w [T,k] f32, row_off [E+1] i32, src [T*k] i32, row_expert [T*k] i32, inv [T*k] i32).
-std::vector<Tensor> router(Tensor z, Tensor corr, int64_t E, int64_t k) {
+// bias fp32 [NE] is added to the logits; renorm: the chosen weights are divided by their sum (= softmax over the chosen).
+std::vector<Tensor> router(Tensor z, c10::optional<Tensor> corr, int64_t E, int64_t k, c10::optional<Tensor> bias,
+                           bool renorm) {
   want(z, torch::kFloat32, "router z");
-  want(corr, torch::kFloat32, "router correction");
-  TORCH_CHECK(z.dim() == 2 && corr.numel() == z.size(1) && E >= 0 && E <= z.size(1) && k >= 1 && k <= z.size(1) &&
+  if (corr.has_value()) want(*corr, torch::kFloat32, "router correction");
+  if (bias.has_value()) want(*bias, torch::kFloat32, "router bias");
+  TORCH_CHECK(z.dim() == 2 && (!corr.has_value() || corr->numel() == z.size(1)) &&
+                  (!bias.has_value() || bias->numel() == z.size(1)) && E >= 0 && E <= z.size(1) && k >= 1 && k <= z.size(1) &&
                   z.size(1) <= r32_router_max_outputs(), "router: shapes disagree");
   const int T = (int)z.size(0), NE = (int)z.size(1);
   auto oi = z.options().dtype(torch::kInt32);
@@ -541,7 +566,8 @@ std::vector<Tensor> router(Tensor z, Tensor corr, int64_t E, int64_t k) {
   Tensor zeroed = torch::zeros({Ec + 2 * (int64_t)T * k}, oi);  // counts | src | row_expert: one fill
   Tensor counts = zeroed.narrow(0, 0, Ec), src = zeroed.narrow(0, Ec, T * k), row_expert = zeroed.narrow(0, Ec + T * k, T * k);
   Tensor row_off = torch::empty({E + 1}, oi), inv = torch::empty({T * k}, oi);
-  done(r32_router(z.data_ptr<float>(), corr.data_ptr<float>(), T, NE, (int)E, (int)k, ids.data_ptr<int>(), w.data_ptr<float>(),
+  done(r32_router(z.data_ptr<float>(), corr.has_value() ? corr->data_ptr<float>() : nullptr,
+                  bias.has_value() ? bias->data_ptr<float>() : nullptr, renorm ? 1 : 0, T, NE, (int)E, (int)k, ids.data_ptr<int>(), w.data_ptr<float>(),
                   counts.data_ptr<int>(), rank.data_ptr<int>(), row_off.data_ptr<int>(), src.data_ptr<int>(),
                   row_expert.data_ptr<int>(), inv.data_ptr<int>(), stream()), "router");
   if (T == 0) row_off.zero_();
@@ -569,7 +595,8 @@ Tensor expert_rows(Tensor h, Tensor src, Tensor row_expert, Tensor row_off, Tens
 }
 
 // out fp32 [T, d] = sum_j w[t][j] * (inv[t k + j] >= 0 ? Y[inv] : h[t])
-Tensor moe_combine(Tensor Y, Tensor inv, Tensor w, Tensor h) {
+// add: rows [T, d] of h's dtype added to every token's sum (a shared expert's result), or absent
+Tensor moe_combine(Tensor Y, Tensor inv, Tensor w, Tensor h, c10::optional<Tensor> add) {
   const int f = act_f32(h, "moe_combine h"), fy = act_f32(Y, "moe_combine Y");
   const int ldh = row_stride(h, "moe_combine h");
   want(inv, torch::kInt32, "moe_combine inv");
@@ -578,9 +605,104 @@ Tensor moe_combine(Tensor Y, Tensor inv, Tensor w, Tensor h) {
   TORCH_CHECK(w.dim() == 2 && w.size(0) == T && inv.numel() == w.numel() && Y.is_contiguous() && Y.dim() == 2 && Y.size(1) == d,
               "moe_combine: shapes disagree");
   Tensor out = torch::empty({T, d}, h.options().dtype(torch::kFloat32));
+  const void* ap = nullptr;
+  int lda = 0;
+  if (add.has_value()) {
+    TORCH_CHECK(add->is_cuda() && add->scalar_type() == h.scalar_type() && add->size(0) == T && add->size(1) == d,
+                "moe_combine: add [T, d] of h's dtype");
+    lda = row_stride(*add, "moe_combine add");
+    ap = add->data_ptr();
+  }
   done(r32_moe_combine(Y.data_ptr(), fy, inv.data_ptr<int>(), w.data_ptr<float>(), h.data_ptr(), ldh, T, (int)w.size(1),
-                       out.data_ptr<float>(), d, f, stream()), "moe_combine");
+                       out.data_ptr<float>(), d, ap, lda, f, stream()), "moe_combine");
   return out;
+}
+
+// Low-rank attention, cache side: proj rows [dq (Cq) | c (C) | rotated key part (R) | ...]; cq [T, Cq] receives the
+// normalised query latent; the normalised c and the rotated part go to the K row (zeros up to nk), c again to the V row.
+void latent_kv_write(Tensor proj, int64_t Cq, int64_t C, int64_t R, Tensor wq, Tensor wc, Tensor freq, double mult,
+                     Tensor positions, Tensor slots, Tensor cq, Tensor k_cache, Tensor v_cache, double eps) {
+  const int f = act_f32(proj, "latent_kv_write proj");
+  const int ldp = row_stride(proj, "latent_kv_write proj"), ldq = row_stride(cq, "latent_kv_write cq");
+  want(wq, torch::kFloat32, "latent_kv_write wq");
+  want(wc, torch::kFloat32, "latent_kv_write wc");
+  want(freq, torch::kFloat32, "latent_kv_write freq");
+  want(positions, torch::kInt32, "latent_kv_write positions");
+  want(slots, torch::kInt32, "latent_kv_write slots");
+  int NB, BS, nk, nv;
+  cache_layout(k_cache, v_cache, NB, BS, nk, nv, "latent_kv_write");
+  const int T = (int)proj.size(0);
+  TORCH_CHECK(k_cache.scalar_type() == proj.scalar_type() && v_cache.scalar_type() == proj.scalar_type() &&
+                  cq.scalar_type() == proj.scalar_type() && cq.is_cuda() && k_cache.is_cuda() && v_cache.is_cuda(),
+              "latent_kv_write: one activation dtype");
+  TORCH_CHECK(Cq >= 1 && C >= 1 && R >= 0 && R % 2 == 0 && proj.size(1) >= Cq + C + R && cq.size(0) == T && cq.size(1) == Cq &&
+                  wq.numel() == Cq && wc.numel() == C && freq.numel() == R / 2 && positions.numel() == T && slots.numel() == T &&
+                  nk >= C + R && nv >= C, "latent_kv_write: shapes disagree");
+  done(r32_latent_kv_write(proj.data_ptr(), ldp, (int)Cq, (int)C, (int)R, wq.data_ptr<float>(), wc.data_ptr<float>(),
+                           freq.data_ptr<float>(), (float)mult, positions.data_ptr<int>(), slots.data_ptr<int>(), cq.data_ptr(),
+                           ldq, k_cache.data_ptr(), v_cache.data_ptr(), (long long)k_cache.stride(0),
+                           (long long)v_cache.stride(0), BS, nk, nv, (float)eps, T, f, stream()), "latent_kv_write");
+}
+
+// q [T, H (D + R)] up-projected query rows; qn fp32 [H, T, C] their unrotated parts moved into the latent's space;
+// out fp32 [T, H, Dk] = [qn scale | rot(q_rot) scale | 0]
+void latent_q_rows(Tensor q, int64_t D, int64_t R, Tensor qn, Tensor freq, double mult, double scale, Tensor positions,
+                   Tensor out, int64_t H) {
+  const int f = act_f32(q, "latent_q_rows q");
+  const int ldq = row_stride(q, "latent_q_rows q");
+  want(qn, torch::kFloat32, "latent_q_rows qn");
+  want(freq, torch::kFloat32, "latent_q_rows freq");
+  want(positions, torch::kInt32, "latent_q_rows positions");
+  want(out, torch::kFloat32, "latent_q_rows out");
+  const int T = (int)q.size(0);
+  TORCH_CHECK(qn.dim() == 3 && qn.size(0) == H && qn.size(1) == T && out.dim() == 3 && out.size(0) == T && out.size(1) == H &&
+                  q.size(1) == H * (D + R) && R % 2 == 0 && freq.numel() == R / 2 && positions.numel() == T &&
+                  out.size(2) >= qn.size(2) + R, "latent_q_rows: shapes disagree");
+  done(r32_latent_q_rows(q.data_ptr(), ldq, (int)D, (int)R, qn.data_ptr<float>(), (int)qn.size(2), freq.data_ptr<float>(),
+                         (float)mult, (float)scale, positions.data_ptr<int>(), out.data_ptr<float>(), (int)H, (int)out.size(2), T,
+                         f, stream()), "latent_q_rows");
+}
+
+int64_t retention_max_dim() { return r32_retention_max_dim(); }
+
+// proj rows with q at column 0 and k at k_off (H heads of D each); v rows [T, H Dv] (a column slice is fine); state fp32
+// [slots, H, D, Dv]; out fp32 [T, H Dv]
+void retention(Tensor proj, int64_t k_off, Tensor v, Tensor freq, double mult, int64_t rd, Tensor decay, Tensor state, Tensor cu,
+               Tensor item_slot, Tensor positions, Tensor out, int64_t H) {
+  const int f = act_f32(proj, "retention proj");
+  const int ldp = row_stride(proj, "retention proj"), ldv = row_stride(v, "retention v"), ldo = row_stride(out, "retention out");
+  want(freq, torch::kFloat32, "retention freq");
+  want(decay, torch::kFloat32, "retention decay");
+  want(cu, torch::kInt32, "retention cu");
+  want(item_slot, torch::kInt32, "retention item_slot");
+  want(positions, torch::kInt32, "retention positions");
+  want_dev(state, torch::kFloat32, "retention state");
+  want_dev(out, torch::kFloat32, "retention out");
+  TORCH_CHECK(v.is_cuda() && v.scalar_type() == proj.scalar_type(), "retention: v of proj's dtype");
+  TORCH_CHECK(state.dim() == 4 && state.size(1) == H && state.stride(3) == 1 && state.stride(2) == state.size(3) &&
+                  state.stride(1) == state.size(2) * state.size(3), "retention: state [slots, H, D, Dv]");
+  const int D = (int)state.size(2), Dv = (int)state.size(3), T = (int)proj.size(0);
+  TORCH_CHECK(k_off >= H * D && proj.size(1) >= k_off + H * D && v.size(0) == T && v.size(1) == H * Dv && out.size(0) == T &&
+                  out.size(1) == H * Dv && rd >= 0 && rd % 2 == 0 && rd <= D && freq.numel() == rd / 2 && decay.numel() == H &&
+                  positions.numel() == T && cu.numel() == item_slot.numel() + 1 && D <= r32_retention_max_dim(),
+              "retention: shapes disagree");
+  Tensor qk = torch::empty({T, 2 * H * D}, out.options());
+  done(r32_retention_prep(proj.data_ptr(), ldp, (int)k_off, freq.data_ptr<float>(), (float)mult, positions.data_ptr<int>(),
+                          qk.data_ptr<float>(), T, (int)H, D, (int)rd, 1.0f / std::sqrt((float)D), f, stream()),
+       "retention_prep");
+  done(r32_retention(qk.data_ptr<float>(), v.data_ptr(), ldv, decay.data_ptr<float>(), state.data_ptr<float>(),
+                     (long long)state.stride(0), cu.data_ptr<int>(), item_slot.data_ptr<int>(), positions.data_ptr<int>(),
+                     out.data_ptr<float>(), ldo, (int)item_slot.numel(), (int)H, D, Dv, f, stream()), "retention");
+}
+
+// in rows [gate (n) | up (n)], out rows of n; mode 0 silu(g) u, 1 the clamped unit g' sigmoid(alpha g') (u' + 1)
+void glu(Tensor in, Tensor out, int64_t mode, double alpha, double limit) {
+  const int f = act_f32(in, "glu in");
+  const int ldi = row_stride(in, "glu in"), ldo = row_stride(out, "glu out");
+  TORCH_CHECK(out.is_cuda() && out.scalar_type() == in.scalar_type() && in.size(0) == out.size(0) && in.size(1) == 2 * out.size(1) &&
+                  (mode == 0 || mode == 1), "glu: shapes or dtypes disagree");
+  done(r32_glu(in.data_ptr(), ldi, out.data_ptr(), ldo, (int)in.size(0), (int)out.size(1), (int)mode, (float)alpha, (float)limit,
+               f, stream()), "glu");
 }
 
 }  // namespace
@@ -613,4 +735,9 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
   m.def("router_max_outputs", &router_max_outputs);
   m.def("expert_rows", &expert_rows);
   m.def("moe_combine", &moe_combine);
+  m.def("latent_kv_write", &latent_kv_write);
+  m.def("latent_q_rows", &latent_q_rows);
+  m.def("retention", &retention);
+  m.def("retention_max_dim", &retention_max_dim);
+  m.def("glu", &glu);
 }

@@ -16,7 +16,8 @@ namespace {
 constexpr int kMaxPerLane = 8;  // router outputs per lane: NE <= 512
 
 template <int PER>
-__global__ void router_topk_kernel(const float* __restrict__ z, const float* __restrict__ corr, int NE, int E, int k,
+__global__ void router_topk_kernel(const float* __restrict__ z, const float* __restrict__ corr,
+                                   const float* __restrict__ bias, int renorm, int NE, int E, int k,
                                    int* __restrict__ ids, float* __restrict__ wts, int* __restrict__ counts,
                                    int* __restrict__ rank, int T) {
   const int t = blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6);
@@ -28,7 +29,7 @@ __global__ void router_topk_kernel(const float* __restrict__ z, const float* __r
 #pragma unroll
   for (int i = 0; i < PER; ++i) {
     const int e = lane + 64 * i;
-    v[i] = e < NE ? zr[e] : -INFINITY;
+    v[i] = e < NE ? zr[e] + (bias ? bias[e] : 0.f) : -INFINITY;
     m = fmaxf(m, v[i]);
   }
   m = wave_max(m);
@@ -44,8 +45,9 @@ __global__ void router_topk_kernel(const float* __restrict__ z, const float* __r
   for (int i = 0; i < PER; ++i) {
     const int e = lane + 64 * i;
     v[i] = v[i] / sum;
-    c[i] = e < NE ? v[i] + corr[e] : -INFINITY;
+    c[i] = e < NE ? v[i] + (corr ? corr[e] : 0.f) : -INFINITY;
   }
+  float chosen = 0.f;
   for (int j = 0; j < k; ++j) {
     float best = -INFINITY;
     int bi = 0x7fffffff;
@@ -66,17 +68,21 @@ __global__ void router_topk_kernel(const float* __restrict__ z, const float* __r
     for (int i = 0; i < PER; ++i)
       if (lane + 64 * i == bi) sc = v[i], c[i] = -INFINITY;
     sc = wave_sum(sc);
+    chosen += sc;
     if (lane == 0) {
       ids[(size_t)t * k + j] = bi;
       wts[(size_t)t * k + j] = sc;
       rank[(size_t)t * k + j] = bi < E ? atomicAdd(counts + bi, 1) : -1;
     }
   }
+  if (renorm && lane == 0)  // weights = softmax over the chosen outputs only
+    for (int j = 0; j < k; ++j) wts[(size_t)t * k + j] /= chosen;
 }
 
 // Few router outputs (NE <= NMAX): one THREAD per token, the scores in registers.
 template <int NMAX>
-__global__ void router_topk_thread_kernel(const float* __restrict__ z, const float* __restrict__ corr, int NE, int E, int k,
+__global__ void router_topk_thread_kernel(const float* __restrict__ z, const float* __restrict__ corr,
+                                          const float* __restrict__ bias, int renorm, int NE, int E, int k,
                                           int* __restrict__ ids, float* __restrict__ wts, int* __restrict__ counts,
                                           int* __restrict__ rank, int T) {
   const int t0 = blockIdx.x * blockDim.x + threadIdx.x;
@@ -87,7 +93,7 @@ __global__ void router_topk_thread_kernel(const float* __restrict__ z, const flo
   float m = -INFINITY;
 #pragma unroll
   for (int i = 0; i < NMAX; ++i) {
-    v[i] = i < NE ? zr[i] : -INFINITY;
+    v[i] = i < NE ? zr[i] + (bias ? bias[i] : 0.f) : -INFINITY;
     m = fmaxf(m, v[i]);
   }
   float sum = 0.f;
@@ -99,8 +105,9 @@ __global__ void router_topk_thread_kernel(const float* __restrict__ z, const flo
 #pragma unroll
   for (int i = 0; i < NMAX; ++i) {
     v[i] = v[i] / sum;
-    c[i] = i < NE ? v[i] + corr[i] : -INFINITY;
+    c[i] = i < NE ? v[i] + (corr ? corr[i] : 0.f) : -INFINITY;
   }
+  float chosen = 0.f;
   for (int j = 0; j < k; ++j) {
     float best = -INFINITY, sc = 0.f;
     int bi = 0;
@@ -110,6 +117,7 @@ __global__ void router_topk_thread_kernel(const float* __restrict__ z, const flo
 #pragma unroll
     for (int i = 0; i < NMAX; ++i)
       if (i == bi) c[i] = -INFINITY;
+    chosen += sc;
     if (live) {
       ids[(size_t)t * k + j] = bi;
       wts[(size_t)t * k + j] = sc;
@@ -128,6 +136,8 @@ __global__ void router_topk_thread_kernel(const float* __restrict__ z, const flo
     }
     if (live) rank[(size_t)t * k + j] = rk;
   }
+  if (renorm && live)  // weights = softmax over the chosen outputs only
+    for (int j = 0; j < k; ++j) wts[(size_t)t * k + j] /= chosen;
 }
 
 __global__ void router_offsets_kernel(const int* __restrict__ counts, int E, int* __restrict__ row_off) {
@@ -199,10 +209,11 @@ __global__ void __launch_bounds__(256) expert_rows_kernel(const AT* __restrict__
 
 template <typename AT, typename YT>
 __global__ void moe_combine_kernel(const YT* __restrict__ Y, const int* __restrict__ inv, const float* __restrict__ wts,
-                                   const AT* __restrict__ h, int ldh, int k, float* __restrict__ out, int d) {
+                                   const AT* __restrict__ h, int ldh, int k, float* __restrict__ out, int d,
+                                   const AT* __restrict__ add, int lda) {
   const int t = blockIdx.x;
   for (int c = threadIdx.x; c < d; c += blockDim.x) {
-    float s = 0.f;
+    float s = add ? Elem<AT>::ld(add + (size_t)t * lda + c) : 0.f;
     for (int j = 0; j < k; ++j) {
       const int r = inv[(size_t)t * k + j];
       const float v = r >= 0 ? Elem<YT>::ld(Y + (size_t)r * d + c) : Elem<AT>::ld(h + (size_t)t * ldh + c);
@@ -215,10 +226,11 @@ __global__ void moe_combine_kernel(const YT* __restrict__ Y, const int* __restri
 // four columns per thread (d a multiple of four, aligned bases)
 template <typename AT, typename YT>
 __global__ void moe_combine_vec_kernel(const YT* __restrict__ Y, const int* __restrict__ inv, const float* __restrict__ wts,
-                                       const AT* __restrict__ h, int ldh, int k, float* __restrict__ out, int d) {
+                                       const AT* __restrict__ h, int ldh, int k, float* __restrict__ out, int d,
+                                       const AT* __restrict__ add, int lda) {
   const int t = blockIdx.x;
   for (int c = threadIdx.x * 4; c < d; c += blockDim.x * 4) {
-    float4v s = float4v{0.f, 0.f, 0.f, 0.f};
+    float4v s = add ? Vec4<AT>::ld(add + (size_t)t * lda + c) : float4v{0.f, 0.f, 0.f, 0.f};
     for (int j = 0; j < k; ++j) {
       const int r = inv[(size_t)t * k + j];
       const float4v v = r >= 0 ? Vec4<YT>::ld(Y + (size_t)r * d + c) : Vec4<AT>::ld(h + (size_t)t * ldh + c);
@@ -236,13 +248,16 @@ using namespace lwc;
 extern "C" int r32_router_max_outputs() { return 64 * kMaxPerLane; }
 
 // counts must be zero on entry (E ints)
-extern "C" int r32_router(const float* z, const float* corr, int T, int NE, int E, int k, int* ids, float* wts, int* counts,
-                          int* rank, int* row_off, int* src, int* row_expert, int* inv, hipStream_t s) {
+// corr (added to the softmax for the choice only) and bias (added to the logits) may be null; renorm != 0: the chosen
+// weights are divided by their sum
+extern "C" int r32_router(const float* z, const float* corr, const float* bias, int renorm, int T, int NE, int E, int k,
+                          int* ids, float* wts, int* counts, int* rank, int* row_off, int* src, int* row_expert, int* inv,
+                          hipStream_t s) {
   if (T <= 0) return 0;
   if (NE > 64 * kMaxPerLane || k < 1 || k > NE || E > NE) return -1;
-  if (NE <= 16) router_topk_thread_kernel<16><<<(T + 63) / 64, 64, 0, s>>>(z, corr, NE, E, k, ids, wts, counts, rank, T);
-  else if (NE <= 64) router_topk_kernel<1><<<(T + 3) / 4, 256, 0, s>>>(z, corr, NE, E, k, ids, wts, counts, rank, T);
-  else router_topk_kernel<kMaxPerLane><<<(T + 3) / 4, 256, 0, s>>>(z, corr, NE, E, k, ids, wts, counts, rank, T);
+  if (NE <= 16) router_topk_thread_kernel<16><<<(T + 63) / 64, 64, 0, s>>>(z, corr, bias, renorm, NE, E, k, ids, wts, counts, rank, T);
+  else if (NE <= 64) router_topk_kernel<1><<<(T + 3) / 4, 256, 0, s>>>(z, corr, bias, renorm, NE, E, k, ids, wts, counts, rank, T);
+  else router_topk_kernel<kMaxPerLane><<<(T + 3) / 4, 256, 0, s>>>(z, corr, bias, renorm, NE, E, k, ids, wts, counts, rank, T);
   router_offsets_kernel<<<1, 64, 0, s>>>(counts, E, row_off);
   const int total = T * k;
   router_scatter_kernel<<<(total + 255) / 256, 256, 0, s>>>(ids, rank, row_off, E, k, src, row_expert, inv, total);
@@ -266,27 +281,28 @@ extern "C" int r32_expert_rows(const void* h, int ldh, const int* src, const int
   return 0;
 }
 
+// add: rows of the activation type added to every token's sum (a shared expert), or null
 extern "C" int r32_moe_combine(const void* Y, int y_f32, const int* inv, const float* wts, const void* h, int ldh, int T,
-                               int k, float* out, int d, int f32, hipStream_t s) {
+                               int k, float* out, int d, const void* add, int lda, int f32, hipStream_t s) {
   if (T <= 0) return 0;
-  if (d % 4 == 0 && ldh % 4 == 0 && aligned_to(Y, y_f32 ? 16 : 8) && aligned_to(h, f32 ? 16 : 8) && aligned_to(out, 16)) {
+  if (d % 4 == 0 && ldh % 4 == 0 && lda % 4 == 0 && aligned_to(add, f32 ? 16 : 8) && aligned_to(Y, y_f32 ? 16 : 8) && aligned_to(h, f32 ? 16 : 8) && aligned_to(out, 16)) {
     if (f32 && y_f32)
-      moe_combine_vec_kernel<float, float><<<T, 256, 0, s>>>((const float*)Y, inv, wts, (const float*)h, ldh, k, out, d);
+      moe_combine_vec_kernel<float, float><<<T, 256, 0, s>>>((const float*)Y, inv, wts, (const float*)h, ldh, k, out, d, (const float*)add, lda);
     else if (!f32 && y_f32)
-      moe_combine_vec_kernel<bf16_t, float><<<T, 256, 0, s>>>((const float*)Y, inv, wts, (const bf16_t*)h, ldh, k, out, d);
+      moe_combine_vec_kernel<bf16_t, float><<<T, 256, 0, s>>>((const float*)Y, inv, wts, (const bf16_t*)h, ldh, k, out, d, (const bf16_t*)add, lda);
     else if (!f32 && !y_f32)
-      moe_combine_vec_kernel<bf16_t, bf16_t><<<T, 256, 0, s>>>((const bf16_t*)Y, inv, wts, (const bf16_t*)h, ldh, k, out, d);
+      moe_combine_vec_kernel<bf16_t, bf16_t><<<T, 256, 0, s>>>((const bf16_t*)Y, inv, wts, (const bf16_t*)h, ldh, k, out, d, (const bf16_t*)add, lda);
     else
       return -1;
     LWC_CHECK_LAUNCH();
     return 0;
   }
   if (f32 && y_f32)
-    moe_combine_kernel<float, float><<<T, 256, 0, s>>>((const float*)Y, inv, wts, (const float*)h, ldh, k, out, d);
+    moe_combine_kernel<float, float><<<T, 256, 0, s>>>((const float*)Y, inv, wts, (const float*)h, ldh, k, out, d, (const float*)add, lda);
   else if (!f32 && y_f32)
-    moe_combine_kernel<bf16_t, float><<<T, 256, 0, s>>>((const float*)Y, inv, wts, (const bf16_t*)h, ldh, k, out, d);
+    moe_combine_kernel<bf16_t, float><<<T, 256, 0, s>>>((const float*)Y, inv, wts, (const bf16_t*)h, ldh, k, out, d, (const bf16_t*)add, lda);
   else if (!f32 && !y_f32)
-    moe_combine_kernel<bf16_t, bf16_t><<<T, 256, 0, s>>>((const bf16_t*)Y, inv, wts, (const bf16_t*)h, ldh, k, out, d);
+    moe_combine_kernel<bf16_t, bf16_t><<<T, 256, 0, s>>>((const bf16_t*)Y, inv, wts, (const bf16_t*)h, ldh, k, out, d, (const bf16_t*)add, lda);
   else
     return -1;
   LWC_CHECK_LAUNCH();

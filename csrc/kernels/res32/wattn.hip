@@ -61,15 +61,15 @@ template <> struct KLoad<float> {
   static LWC_DEVICE void st(float* p, float v) { *p = v; }
 };
 
-constexpr int kMaxSlots = 4;  // value dimension <= 256
+constexpr int kMaxSlots = 8;  // value dimension <= 512
 
 template <typename CT>
 __global__ void __launch_bounds__(64)
 window_attn_kernel(const float* __restrict__ q, const CT* __restrict__ k_cache, const CT* __restrict__ v_cache,
                    long long kb_stride, long long vb_stride, int block_size, const int* __restrict__ positions,
                    const int* __restrict__ cu_q, int n_items, const int* __restrict__ block_tables, int bt_width,
-                   const float* __restrict__ r1, const float* __restrict__ r2, int window, CT* __restrict__ out,
-                   int ldo, int H, int G, int D, int Dv) {
+                   const float* __restrict__ r1, const float* __restrict__ r2, const float* __restrict__ sink, int window,
+                   CT* __restrict__ out, int ldo, int H, int G, int D, int Dv) {
   extern __shared__ float q_s[];  // [D]
   __shared__ float p_s[64];
   __shared__ long long vo_s[64];
@@ -95,7 +95,9 @@ window_attn_kernel(const float* __restrict__ q, const CT* __restrict__ k_cache, 
     while (DvP < Dv) DvP <<= 1;
   }
   const int kpar = 64 / DvP, dvl = lane % DvP, kp = lane / DvP;
-  float o[kMaxSlots] = {0.f, 0.f, 0.f, 0.f};
+  float o[kMaxSlots];
+#pragma unroll
+  for (int ns = 0; ns < kMaxSlots; ++ns) o[ns] = 0.f;
   float m = -INFINITY, l = 0.f;
   const int j_lo = max(0, i - window + 1);
   for (int j0 = j_lo; j0 <= i; j0 += 64) {
@@ -133,6 +135,12 @@ window_attn_kernel(const float* __restrict__ q, const CT* __restrict__ k_cache, 
     }
   }
   for (int off = DvP; off < 64; off <<= 1) o[0] += __shfl_xor(o[0], off, 64);
+  if (sink) {  // a sink: exp(sink_h) joins the denominator; it has no key and no value
+    const float sk = sink[h], mf = fmaxf(m, sk), a = expf(m - mf);
+    l = l * a + expf(sk - mf);
+#pragma unroll
+    for (int ns = 0; ns < kMaxSlots; ++ns) o[ns] *= a;
+  }
   if (kp == 0) {
     const float inv = 1.0f / l;
     CT* orow = out + (size_t)t * ldo + (size_t)h * Dv;
@@ -151,8 +159,8 @@ using namespace lwc;
 
 extern "C" int r32_window_attn(const float* q, const void* k_cache, const void* v_cache, long long kb_stride,
                                long long vb_stride, int block_size, const int* positions, const int* cu_q, int n_items,
-                               const int* block_tables, int bt_width, const float* r1, const float* r2, int window,
-                               void* out, int ldo, int T, int H, int G, int D, int Dv, int f32, hipStream_t s) {
+                               const int* block_tables, int bt_width, const float* r1, const float* r2, const float* sink,
+                               int window, void* out, int ldo, int T, int H, int G, int D, int Dv, int f32, hipStream_t s) {
   if (T <= 0) return 0;
   if (Dv > 64 * kMaxSlots || D > 8192 || H % G != 0) return -1;
   const dim3 grid(T, H);
@@ -160,11 +168,11 @@ extern "C" int r32_window_attn(const float* q, const void* k_cache, const void* 
   if (f32)
     window_attn_kernel<float><<<grid, 64, shm, s>>>(q, (const float*)k_cache, (const float*)v_cache, kb_stride, vb_stride,
                                                     block_size, positions, cu_q, n_items, block_tables, bt_width, r1, r2,
-                                                    window, (float*)out, ldo, H, G, D, Dv);
+                                                    sink, window, (float*)out, ldo, H, G, D, Dv);
   else
     window_attn_kernel<bf16_t><<<grid, 64, shm, s>>>(q, (const bf16_t*)k_cache, (const bf16_t*)v_cache, kb_stride,
                                                      vb_stride, block_size, positions, cu_q, n_items, block_tables,
-                                                     bt_width, r1, r2, window, (bf16_t*)out, ldo, H, G, D, Dv);
+                                                     bt_width, r1, r2, sink, window, (bf16_t*)out, ldo, H, G, D, Dv);
   return (int)hipGetLastError();
 }
 

@@ -360,8 +360,209 @@ class MerudraConfig:
         return n
 
 
+# ------------------------------------------------------------------ Limatar
+@dataclass(frozen=True)
+class RotarySpec:
+    """Rotation by position of the first ``dims`` entries of a head: pair i turns by position * f_i, f_i =
+    base^(-2i/dims).  ``scaling`` (factor, original, fast, slow) stretches the slow pairs (frequency blending over a
+    ramp of the pair index) and multiplies the cos / sin tables by 0.1 ln(factor) + 1."""
+    dims: int
+    base: float
+    scaling: Optional[Tuple[float, float, float, float]] = None   # factor, original, fast, slow
+
+    def scaling_dict(self) -> Optional[dict]:
+        if self.scaling is None:
+            return None
+        f, o, a, b = self.scaling
+        return {"factor": f, "original": o, "fast": a, "slow": b}
+
+    @classmethod
+    def from_dict(cls, r: dict) -> "RotarySpec":
+        sc = r.get("scaling")
+        return cls(dims=int(r["dims"]), base=float(r["base"]),
+                   scaling=None if not sc else (float(sc["factor"]), float(sc["original"]), float(sc["fast"]),
+                                                float(sc["slow"])))
+
+
+@dataclass(frozen=True)
+class LatentAttentionSpec:
+    """Causal softmax attention whose queries and keys / values pass through low-rank latents (``q_rank``,
+    ``kv_rank``); per head ``dim`` unrotated and ``rot_dim`` rotated query / key entries (the rotated key part is one
+    vector for all heads, pairs interleaved), values of ``vdim``; a learned sink per head in the softmax's
+    denominator; a sigmoid output gate."""
+    heads: int
+    dim: int
+    rot_dim: int
+    vdim: int
+    q_rank: int
+    kv_rank: int
+    scale: float
+    rot: RotarySpec
+
+    kv_heads = 1   # one cached row (latent + rotated part) serves every head
+
+    @property
+    def nq(self) -> int:
+        return self.heads * (self.dim + self.rot_dim)
+
+    @property
+    def nv(self) -> int:
+        return self.heads * self.vdim
+
+
+@dataclass(frozen=True)
+class RetentionSpec:
+    """Linear attention with a fixed decay per head: S <- a_h S + k v^T, o = S^T q; q, k rotated ("rotate half"
+    pairing), per-head unit RMS on o, a silu gate."""
+    heads: int
+    dim: int
+    vdim: int
+    decay: Tuple[float, ...]
+    rot: RotarySpec
+
+    kv_heads = 0
+
+    @property
+    def nq(self) -> int:
+        return self.heads * self.dim
+
+    @property
+    def nv(self) -> int:
+        return self.heads * self.vdim
+
+
+@dataclass(frozen=True)
+class ClampedGluSpec:
+    """Dense feed-forward W_down (g' sigmoid(alpha g') (u' + 1)) with g' = min(g, limit), u' = clamp(u, +-limit)."""
+    ff: int
+    limit: float
+    alpha: float = 1.702   # fixed by the design
+
+
+@dataclass(frozen=True)
+class TopkExpertsSpec:
+    """Routed experts (silu-gated, no biases): the ``top`` largest router logits (+ bias) choose, the weights are the
+    softmax over the chosen logits; ``shared_ff`` > 0: one more expert of that width runs for every token."""
+    experts: int
+    top: int
+    ff: int
+    shared_ff: int
+
+
+@dataclass(frozen=True)
+class LimatarLayerSpec:
+    type: str                 # "latent_attention" | "retention"
+    mixer: object             # LatentAttentionSpec | RetentionSpec
+    mlp: object               # ClampedGluSpec | TopkExpertsSpec | None
+
+
+@dataclass(frozen=True)
+class LimatarConfig:
+    """Limatar: an fp32 residual stream with a norm before AND after every sublayer (weights stored around zero),
+    mixers = low-rank attention with sinks or retention, feed-forwards = a clamped gated unit or routed experts with a
+    shared expert, a span of layers that runs several times in a row with the same weights (every pass has its own
+    cache and state), output weights tied to the embedding."""
+    name: str
+    vocab_size: int
+    hidden: int
+    layer_specs: Tuple[LimatarLayerSpec, ...]
+    norm_eps: float
+    loop_start: int = 0
+    loop_stop: int = 0
+    loop_times: int = 1
+    bos_token_id: int = 1
+    eos_token_id: int = 2
+
+    architecture = "Limatar"
+    num_experts = 0   # the engine's expert-parallel planning does not apply
+
+    @property
+    def runs(self) -> Tuple[int, ...]:
+        """The layer index of every layer run, in execution order (the looped span repeated in a row)."""
+        n = len(self.layer_specs)
+        a, b = self.loop_start, self.loop_stop
+        return tuple(range(a)) + tuple(range(a, b)) * self.loop_times + tuple(range(b, n))
+
+    @property
+    def layers(self) -> int:
+        return len(self.runs)
+
+    @property
+    def heads(self) -> int:
+        return max(L.mixer.heads for L in self.layer_specs)
+
+    @property
+    def kv_heads(self) -> int:
+        return 1
+
+    @property
+    def head_dim(self) -> int:
+        return max(L.mixer.dim for L in self.layer_specs)
+
+    @classmethod
+    def from_dict(cls, c: dict, name: str = "limatar") -> "LimatarConfig":
+        specs = []
+        for L in c["layers"]:
+            m = L["mixer"]
+            if L["type"] == "latent_attention":
+                rot = RotarySpec.from_dict(m["rot"])
+                mixer = LatentAttentionSpec(heads=int(m["heads"]), dim=int(m["dim"]), rot_dim=int(m["rot_dim"]),
+                                            vdim=int(m["vdim"]), q_rank=int(m["q_rank"]), kv_rank=int(m["kv_rank"]),
+                                            scale=float(m["scale"]), rot=rot)
+                if rot.dims != mixer.rot_dim or rot.dims % 2:
+                    raise ValueError("Limatar: a latent attention layer rotates its whole rot_dim part (an even size)")
+            elif L["type"] == "retention":
+                rot = RotarySpec.from_dict(m["rot"])
+                mixer = RetentionSpec(heads=int(m["heads"]), dim=int(m["dim"]), vdim=int(m["vdim"]),
+                                      decay=tuple(float(a) for a in m["decay"]), rot=rot)
+                if len(mixer.decay) != mixer.heads:
+                    raise ValueError("Limatar: one decay per retention head")
+                if rot.dims % 2 or rot.dims > mixer.dim:
+                    raise ValueError("Limatar: rot.dims must be even and at most dim")
+            else:
+                raise ValueError(f"Limatar: unknown mixer type {L['type']!r}")
+            mlp = L.get("mlp")
+            spec = None
+            if mlp is not None:
+                if mlp.get("kind") == "dense":
+                    spec = ClampedGluSpec(ff=int(mlp["ff"]), limit=float(mlp["limit"]))
+                elif mlp.get("kind") == "moe":
+                    r = mlp["router"]
+                    sh = mlp.get("shared")
+                    spec = TopkExpertsSpec(experts=int(r["experts"]), top=int(r["top"]), ff=int(mlp["expert"]["ff"]),
+                                           shared_ff=int(sh["ff"]) if sh else 0)
+                    if not 1 <= spec.top <= spec.experts:
+                        raise ValueError("Limatar: router.top out of range")
+                else:
+                    raise ValueError(f"Limatar: unknown feed-forward kind {mlp.get('kind')!r}")
+            specs.append(LimatarLayerSpec(L["type"], mixer, spec))
+        lp = c.get("loop") or {}
+        a, b, times = int(lp.get("start", 0)), int(lp.get("stop", 0)), int(lp.get("times", 1))
+        if not (0 <= a <= b <= len(specs)) or times < 1:
+            raise ValueError("Limatar: loop span out of range")
+        return cls(name=name, vocab_size=int(c["vocab"]), hidden=int(c["width"]), layer_specs=tuple(specs),
+                   norm_eps=float(c["norm"]["eps"]), loop_start=a, loop_stop=b, loop_times=times)
+
+    def params(self) -> int:
+        d = self.hidden
+        n = self.vocab_size * d + 2 * d
+        for L in self.layer_specs:
+            m = L.mixer
+            n += 2 * d
+            if L.type == "latent_attention":
+                n += d * (m.q_rank + m.kv_rank + m.rot_dim + m.nv) + m.q_rank + m.kv_rank + m.q_rank * m.nq
+                n += m.kv_rank * m.heads * (m.dim + m.vdim) + m.heads + d * m.nv
+            else:
+                n += d * (2 * m.nq + 2 * m.nv) + d * m.nv
+            if isinstance(L.mlp, ClampedGluSpec):
+                n += 2 * d + 3 * d * L.mlp.ff
+            elif L.mlp is not None:
+                n += 2 * d + (L.mlp.experts * L.mlp.ff + L.mlp.shared_ff) * 3 * d + L.mlp.experts * (d + 1)
+        return n
+
+
 # config.json "architecture" -> config class of the layer-list decoders
-ARCHITECTURES = {"Madipel": MadipelConfig, "Merudra": MerudraConfig}
+ARCHITECTURES = {"Madipel": MadipelConfig, "Merudra": MerudraConfig, "Limatar": LimatarConfig}
 
 
 def load_model_config(model_dir) -> object:

@@ -104,16 +104,18 @@ def distance_bias(r1: torch.Tensor, r2: torch.Tensor, window: int) -> torch.Tens
 def window_attn(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, positions: torch.Tensor,
                 block_tables: torch.Tensor, r1: torch.Tensor, r2: torch.Tensor, window: int, out: torch.Tensor,
                 H: int, G: int, cu_q: Optional[torch.Tensor] = None, k_lens: Optional[torch.Tensor] = None,
-                max_q: int = 0, bias: Optional[torch.Tensor] = None, cores: Optional[bool] = None) -> torch.Tensor:
+                max_q: int = 0, bias: Optional[torch.Tensor] = None, cores: Optional[bool] = None,
+                sink: Optional[torch.Tensor] = None) -> torch.Tensor:
     """Sliding-window attention over the paged cache with the bias -r1_h ln(1 + r2_h (i - j)); ``q`` fp32
     [T, H*D] pre-scaled; row t reads table row t (``cu_q`` None) or the item whose ``cu_q`` range holds t.
     Over a bf16 cache whose sizes the matrix-core kernels are built for, prompt portions run on the portion kernel
     (it wants ``k_lens``, ``max_q`` and the ``bias`` table of :func:`distance_bias`) and decode rows on the
     split-key decode kernel (``bias``); everything else on the general kernel.  ``cores=True`` with ``bias`` None:
-    the matrix-core kernels without a distance bias (r1 = 0: plain causal or windowed softmax attention)."""
+    the matrix-core kernels without a distance bias (r1 = 0: plain causal or windowed softmax attention).
+    ``sink`` (fp32 [H]): exp(sink_h) joins head h's softmax denominator; it has no key and no value."""
     K = kernels()
     bs = k_cache.shape[1]
-    cores = ((bias is not None or bool(cores)) and k_cache.dtype == torch.bfloat16 and bs & (bs - 1) == 0
+    cores = ((bias is not None or bool(cores)) and sink is None and k_cache.dtype == torch.bfloat16 and bs & (bs - 1) == 0
              and K.window_attn_mfma_ok(k_cache.shape[2] // G, v_cache.shape[2] // G))
     if cores and cu_q is None and positions.numel() > 0:
         max_keys = min(int(window), block_tables.shape[1] * k_cache.shape[1])
@@ -123,7 +125,7 @@ def window_attn(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, p
         K.window_attn_mfma(q, k_cache, v_cache, positions, cu_q, k_lens, int(max_q), block_tables, bias, int(window), out,
                            int(H), int(G))
         return out
-    K.window_attn(q, k_cache, v_cache, positions, cu_q, block_tables, r1, r2, int(window), out, int(H), int(G))
+    K.window_attn(q, k_cache, v_cache, positions, cu_q, block_tables, r1, r2, int(window), out, int(H), int(G), sink)
     return out
 
 
@@ -242,12 +244,14 @@ def stack_mix(X: torch.Tensor, coef: torch.Tensor, n: int, out: torch.Tensor) ->
     return out
 
 
-def router(z: torch.Tensor, correction: torch.Tensor, experts: int, top: int):
-    """Softmax router over all outputs of ``z`` (fp32 [T, NE]); the ``top`` largest of softmax + correction are
-    chosen, weighted by their softmax (not renormalised).  Outputs >= ``experts`` are identity experts.  Returns
+def router(z: torch.Tensor, correction: Optional[torch.Tensor], experts: int, top: int,
+           bias: Optional[torch.Tensor] = None, renorm: bool = False):
+    """Softmax router over all outputs of ``z`` (fp32 [T, NE]) + ``bias``; the ``top`` largest of softmax + correction
+    are chosen, weighted by their softmax (``renorm``: divided by the chosen ones' sum, which is the softmax over the
+    chosen logits only).  Outputs >= ``experts`` are identity experts.  Returns
     (ids [T, top], w [T, top], row_off [experts + 1], src [T top], row_expert [T top], inv [T top]): expert-major
     row r holds token src[r] for expert row_expert[r]; choice (t, j) is row inv[t top + j], -1 for an identity."""
-    return tuple(kernels().router(z, correction, int(experts), int(top)))
+    return tuple(kernels().router(z, correction, int(experts), int(top), bias, bool(renorm)))
 
 
 def expert_rows(h: torch.Tensor, src: torch.Tensor, row_expert: torch.Tensor, row_off: torch.Tensor, w_gu: torch.Tensor,
@@ -256,6 +260,78 @@ def expert_rows(h: torch.Tensor, src: torch.Tensor, row_expert: torch.Tensor, ro
     return kernels().expert_rows(h, src, row_expert, row_off, w_gu, w_down)
 
 
-def moe_combine(Y: torch.Tensor, inv: torch.Tensor, w: torch.Tensor, h: torch.Tensor) -> torch.Tensor:
-    """fp32 [T, d]: sum_j w[t, j] * (Y[inv[t, j]] if inv >= 0 else h[t])."""
-    return kernels().moe_combine(Y, inv, w, h)
+def moe_combine(Y: torch.Tensor, inv: torch.Tensor, w: torch.Tensor, h: torch.Tensor,
+                add: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """fp32 [T, d]: sum_j w[t, j] * (Y[inv[t, j]] if inv >= 0 else h[t]) (+ ``add[t]``: a shared expert's rows)."""
+    return kernels().moe_combine(Y, inv, w, h, add)
+
+
+# ------------------------------------------------------------------ rotations, low-rank attention, retention, gated units
+def rope_frequencies(dims: int, base: float, scaling: Optional[dict] = None, device="cuda"):
+    """(f fp32 [dims / 2], m): the rotation frequencies base^(-2i/dims) and the multiplier of the cos / sin tables.
+    ``scaling`` = {factor, original, fast, slow} blends f_i with f_i / factor over a linear ramp of the pair index i
+    between the pairs that turn ``fast`` and ``slow`` times within ``original`` positions, and sets
+    m = 0.1 ln(factor) + 1.  Computed in float64, rounded once."""
+    i = torch.arange(dims // 2, dtype=torch.float64)
+    f = float(base) ** (-2.0 * i / dims)
+    m = 1.0
+    if scaling:
+        factor, orig = float(scaling["factor"]), float(scaling["original"])
+
+        def pair_of(turns: float) -> float:
+            return dims * math.log(orig / (2.0 * math.pi * turns)) / (2.0 * math.log(float(base)))
+
+        lo = max(math.floor(pair_of(float(scaling["fast"]))), 0)
+        hi = min(math.ceil(pair_of(float(scaling["slow"]))), dims - 1)
+        ramp = ((i - lo) / max(hi - lo, 0.001)).clamp(0.0, 1.0)
+        f = f / factor * ramp + f * (1.0 - ramp)
+        m = 0.1 * math.log(factor) + 1.0
+    return f.to(torch.float32).to(device), m
+
+
+def latent_kv_write(proj: torch.Tensor, Cq: int, C: int, R: int, wq: torch.Tensor, wc: torch.Tensor, freq: torch.Tensor,
+                    mult: float, positions: torch.Tensor, slots: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor,
+                    eps: float, cq: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """Cache side of a low-rank attention layer.  ``proj`` rows = [dq (Cq) | c (C) | key part to rotate (R) | ...]:
+    returns cq = dq / rms(dq) * wq ([T, Cq], proj's dtype); writes per token ONE key row [c / rms(c) * wc | rotated
+    part * mult | zeros] and the same normalised c as its value row into the paged cache at ``slots`` (-1: no write).
+    Rotation: entries (2i, 2i + 1) by the angle position * freq[i]."""
+    if cq is None:
+        cq = torch.empty(proj.shape[0], Cq, dtype=proj.dtype, device=proj.device)
+    kernels().latent_kv_write(proj, int(Cq), int(C), int(R), wq, wc, freq, float(mult), positions, slots, cq, k_cache,
+                              v_cache, float(eps))
+    return cq
+
+
+def latent_q_rows(q: torch.Tensor, D: int, R: int, qn: torch.Tensor, freq: torch.Tensor, mult: float, scale: float,
+                  positions: torch.Tensor, H: int, Dk: int) -> torch.Tensor:
+    """fp32 query rows [T, H, Dk] of a low-rank attention layer: per head [qn * scale | rot(q[:, D : D + R]) * mult *
+    scale | 0], ``qn`` fp32 [H, T, C] = the unrotated query parts times the keys' up-projection."""
+    out = torch.empty(q.shape[0], H, Dk, dtype=torch.float32, device=q.device)
+    kernels().latent_q_rows(q, int(D), int(R), qn, freq, float(mult), float(scale), positions, out, int(H))
+    return out
+
+
+def retention(proj: torch.Tensor, k_off: int, v: torch.Tensor, freq: torch.Tensor, mult: float, rot_dims: int,
+              decay: torch.Tensor, state: torch.Tensor, items: StepItems, H: int,
+              out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """Retention over a step's items: per head S <- a_h S + k v^T, o = S^T q (no softmax, no denominator).  q (columns
+    0 ..) and k (columns ``k_off`` ..) of ``proj`` are rotated on their first ``rot_dims`` entries (entry i with
+    i + rot_dims / 2, angle position * freq[i]); k is then multiplied by D^-1/2.  ``v`` [T, H Dv] (a column slice of
+    ``proj`` is fine), ``state`` fp32 [slots, H, D, Dv] (read unless the item starts at position 0, written back).
+    Returns o fp32 [T, H Dv]."""
+    if out is None:
+        out = torch.empty(proj.shape[0], H * state.shape[3], dtype=torch.float32, device=proj.device)
+    kernels().retention(proj, int(k_off), v, freq, float(mult), int(rot_dims), decay, state, items.cu, items.slots,
+                        items.positions, out, int(H))
+    return out
+
+
+def glu(gu: torch.Tensor, out: Optional[torch.Tensor] = None, mode: str = "silu", alpha: float = 1.0,
+        limit: float = 0.0) -> torch.Tensor:
+    """Gated unit over fused rows [gate | up]: ``silu``: silu(g) * u; ``clamped``: g' = min(g, limit), u' = clamp(u,
+    +-limit), g' * sigmoid(alpha g') * (u' + 1)."""
+    if out is None:
+        out = torch.empty(gu.shape[0], gu.shape[1] // 2, dtype=gu.dtype, device=gu.device)
+    kernels().glu(gu, out, 0 if mode == "silu" else 1, float(alpha), float(limit))
+    return out
