@@ -79,6 +79,15 @@ def rotate_half(x, cos, sin):
     return torch.cat([u * c - v * s, v * c + u * s], -1)
 
 
+def sink_softmax(s, sink):
+    """Softmax over the last axis of s [H, ..., keys] whose denominator also holds exp(sink_h): the sink takes weight
+    and gives nothing (rows do not sum to one)."""
+    sk = sink.view([-1] + [1] * (s.dim() - 2))
+    mx = torch.maximum(s.max(-1).values, sk)
+    e = torch.exp(s - mx[..., None])
+    return e / (e.sum(-1) + torch.exp(sk - mx))[..., None]
+
+
 def latent_attention(h, W: Callable[[str], torch.Tensor], m: dict, eps: float):
     """h [T, d] -> [T, d].  ``W(name)`` gives the mixer's tensor '.name' in float64."""
     T = h.shape[0]
@@ -95,13 +104,22 @@ def latent_attention(h, W: Callable[[str], torch.Tensor], m: dict, eps: float):
     v = (c @ W("uv").T).view(T, H, Dv)
     s = (torch.einsum("ihd,jhd->hij", q_nope, k_nope) + torch.einsum("ihr,jr->hij", q_rot, k_rot)) * float(m["scale"])
     s = s.masked_fill(pos[None, :, None] < pos[None, None, :], -math.inf)
-    sink = W("sink")                                                     # [H]
-    mx = torch.maximum(s.max(-1).values, sink[:, None])
-    e = torch.exp(s - mx[..., None])
-    p = e / (e.sum(-1) + torch.exp(sink[:, None] - mx))[..., None]       # the sink takes weight and gives nothing
+    p = sink_softmax(s, W("sink"))
     o = torch.einsum("hij,jhv->ihv", p, v).reshape(T, H * Dv)
     o = o * torch.sigmoid(h @ W("g").T)
     return o @ W("o").T
+
+
+def retention_scan(q, k, v, decay, S=None):
+    """q, k [T, H, D], v [T, H, Dv] -> (o [T, H, Dv], final state [H, D, Dv]): S <- a_h S + k v^T, o = S^T q."""
+    T, H, D = q.shape
+    a = torch.tensor(list(decay), dtype=F64)[:, None, None]
+    S = torch.zeros(H, D, v.shape[-1], dtype=F64) if S is None else S.clone()
+    o = torch.empty(T, H, v.shape[-1], dtype=F64)
+    for t in range(T):
+        S = a * S + k[t][:, :, None] * v[t][:, None, :]
+        o[t] = torch.einsum("hdv,hd->hv", S, q[t])
+    return o, S
 
 
 def retention(h, W, m: dict, eps: float, return_state: bool = False):
@@ -116,23 +134,20 @@ def retention(h, W, m: dict, eps: float, return_state: bool = False):
     q[..., :rd] = rotate_half(q[..., :rd], cos, sin)
     k[..., :rd] = rotate_half(k[..., :rd], cos, sin)
     k = k * D ** -0.5
-    decay = torch.tensor([float(a) for a in m["decay"]], dtype=F64)
-    S = torch.zeros(H, D, Dv, dtype=F64)
-    o = torch.empty(T, H, Dv, dtype=F64)
-    for t in range(T):
-        S = decay[:, None, None] * S + k[t][:, :, None] * v[t][:, None, :]
-        o[t] = torch.einsum("hdv,hd->hv", S, q[t])
+    o, S = retention_scan(q, k, v, [float(a) for a in m["decay"]])
     o = rms_unit(o, eps).reshape(T, H * Dv)
     g = h @ W("g").T
     out = (o * (g * torch.sigmoid(g))) @ W("o").T
     return (out, S) if return_state else out
 
 
+def clamped_unit(g, u, limit: float):
+    g, u = g.clamp(max=limit), u.clamp(-limit, limit)
+    return g * torch.sigmoid(1.702 * g) * (u + 1.0)
+
+
 def dense_ff(h, W, mlp: dict):
-    L = float(mlp["limit"])
-    g = (h @ W("gate").T).clamp(max=L)
-    u = (h @ W("up").T).clamp(-L, L)
-    return (g * torch.sigmoid(1.702 * g) * (u + 1.0)) @ W("down").T
+    return clamped_unit(h @ W("gate").T, h @ W("up").T, float(mlp["limit"])) @ W("down").T
 
 
 def gated_expert(h, gate, up, down):
@@ -192,3 +207,79 @@ def forward(cfg: dict, sd: Dict[str, torch.Tensor], tokens, streams: Optional[li
         if streams is not None:
             streams.append(x.clone())
     return norm_zero_centered(x, w("final.norm"), eps) @ w("embed").T
+
+
+# ------------------------------------------------------------------ small configurations and random weights for tests
+def latent_layer(heads, dim, rot_dim, vdim, q_rank, kv_rank, mlp, scale=None, base=5000.0, scaling=None):
+    rot = {"base": base, "dims": rot_dim}
+    if scaling:
+        rot["scaling"] = scaling
+    return {"type": "latent_attention", "mlp": mlp,
+            "mixer": {"heads": heads, "dim": dim, "rot_dim": rot_dim, "vdim": vdim, "q_rank": q_rank, "kv_rank": kv_rank,
+                      "scale": scale if scale is not None else (dim + rot_dim) ** -0.5, "rot": rot}}
+
+
+def retention_layer(heads, dim, vdim, mlp, rot_dims=None, base=3000.0, decay=None):
+    decay = decay or [1.0 - 2.0 ** (-2 - 1.5 * h) for h in range(heads)]
+    return {"type": "retention", "mlp": mlp,
+            "mixer": {"heads": heads, "dim": dim, "vdim": vdim, "decay": decay,
+                      "rot": {"base": base, "dims": dim if rot_dims is None else rot_dims}}}
+
+
+def dense(ff, limit=1.5):
+    return {"kind": "dense", "ff": ff, "limit": limit}
+
+
+def moe(experts, top, ff, shared=None):
+    m = {"kind": "moe", "expert": {"ff": ff}, "router": {"experts": experts, "top": top}}
+    if shared:
+        m["shared"] = {"ff": shared}
+    return m
+
+
+def make_config(width, vocab, layers, loop=None, eps=1e-5):
+    cfg = {"architecture": "Limatar", "layers": layers, "norm": {"eps": eps}, "vocab": vocab, "width": width}
+    if loop:
+        cfg["loop"] = {"start": loop[0], "stop": loop[1], "times": loop[2]}
+    return cfg
+
+
+def make_weights(cfg: dict, seed: int = 0) -> Dict[str, torch.Tensor]:
+    """bf16 tensors under the names a checkpoint of the design uses."""
+    g = torch.Generator().manual_seed(seed)
+    d, V = int(cfg["width"]), int(cfg["vocab"])
+
+    def mat(o, i, s=1.0):
+        return (torch.randn(o, i, generator=g) * s / math.sqrt(i)).to(torch.bfloat16)
+
+    def vec(n, s=0.1, mean=0.0):
+        return (mean + s * torch.randn(n, generator=g)).to(torch.bfloat16)
+
+    W = {"embed": (0.25 * torch.randn(V, d, generator=g)).to(torch.bfloat16), "embed.norm": vec(d), "final.norm": vec(d)}
+    for i, L in enumerate(cfg["layers"]):
+        p, m = f"l{i}.", L["mixer"]
+        W[p + "norm1"], W[p + "norm1b"] = vec(d), vec(d)
+        H, D, Dv = m["heads"], m["dim"], m["vdim"]
+        if L["type"] == "latent_attention":
+            R, C, Cq = m["rot_dim"], m["kv_rank"], m["q_rank"]
+            W[p + "mix.dq"], W[p + "mix.dq.norm"], W[p + "mix.uq"] = mat(Cq, d), vec(Cq, mean=1.0), mat(H * (D + R), Cq, 2.0)
+            W[p + "mix.dkv"], W[p + "mix.dkv.norm"] = mat(C + R, d), vec(C, mean=1.0)
+            W[p + "mix.uk"], W[p + "mix.uv"], W[p + "mix.sink"] = mat(H * D, C, 2.0), mat(H * Dv, C), vec(H, 1.0)
+        else:
+            W[p + "mix.q"], W[p + "mix.k"], W[p + "mix.v"] = mat(H * D, d), mat(H * D, d), mat(H * Dv, d)
+        W[p + "mix.g"], W[p + "mix.o"] = mat(H * Dv, d), mat(d, H * Dv)
+        e = L.get("mlp")
+        if e is None:
+            continue
+        W[p + "norm2"], W[p + "norm2b"] = vec(d), vec(d)
+        if e["kind"] == "dense":
+            W[p + "mlp.gate"], W[p + "mlp.up"], W[p + "mlp.down"] = mat(e["ff"], d, 2.0), mat(e["ff"], d, 2.0), mat(d, e["ff"])
+        else:
+            ff = e["expert"]["ff"]
+            W[p + "mlp.router"], W[p + "mlp.router.b"] = mat(e["router"]["experts"], d, 3.0), vec(e["router"]["experts"], 0.5)
+            for x in range(e["router"]["experts"]):
+                W[f"{p}mlp.e{x}.gate"], W[f"{p}mlp.e{x}.up"], W[f"{p}mlp.e{x}.down"] = mat(ff, d), mat(ff, d), mat(d, ff)
+            if e.get("shared"):
+                sf = e["shared"]["ff"]
+                W[p + "mlp.shared.gate"], W[p + "mlp.shared.up"], W[p + "mlp.shared.down"] = mat(sf, d), mat(sf, d), mat(d, sf)
+    return W
