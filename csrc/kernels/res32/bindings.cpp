@@ -19,11 +19,13 @@ int r32_window_attn(const float*, const void*, const void*, long long, long long
                     hipStream_t);
 int r32_window_attn_mfma_ok(int, int);
 int r32_window_attn_mfma(const float*, const void*, const void*, long long, long long, int, const int*, const int*,
-                         const int*, int, int, const int*, int, const float*, int, void*, int, int, int, int, int,
+                         const int*, int, int, const int*, int, const float*, const float*, int, void*, int, int, int, int, int,
                          hipStream_t);
+int r32_window_attn_decode_ok(int, int);
 int r32_window_attn_decode_splits(int, int, int, int);
 int r32_window_attn_decode(const float*, const void*, const void*, long long, long long, int, const int*, const int*, int,
-                           const float*, int, float*, float*, int, int, void*, int, int, int, int, int, int, hipStream_t);
+                           const float*, const float*, int, float*, float*, int, int, void*, int, int, int, int, int, int,
+                           hipStream_t);
 int r32_conv_hist(const void*, int, const float*, int, int, float*, long long, const int*, const int*, const int*,
                   const int*, void*, int, void*, int, int, int, int, int, int, int, hipStream_t);
 int r32_conv_hist_update(const void*, int, float*, long long, const int*, const int*, int, int, int, int, hipStream_t);
@@ -239,13 +241,21 @@ void window_attn(Tensor q, Tensor k_cache, Tensor v_cache, Tensor positions, c10
 }
 
 bool window_attn_mfma_ok(int64_t D, int64_t Dv) { return r32_window_attn_mfma_ok((int)D, (int)Dv) != 0; }
+bool window_attn_decode_ok(int64_t D, int64_t Dv) { return r32_window_attn_decode_ok((int)D, (int)Dv) != 0; }
+
+const float* sink_ptr(const c10::optional<Tensor>& sink, int64_t H, const char* name) {
+  if (!sink.has_value()) return nullptr;
+  want(*sink, torch::kFloat32, name);
+  TORCH_CHECK(sink->numel() == H, name, ": sink [H]");
+  return sink->data_ptr<float>();
+}
 
 // Prompt portions on the matrix cores: bf16 caches, q fp32 [T, H*D], bias fp32 [H, window] (the distance bias by
 // i - j), cu_q / k_lens int32 per item (k_lens: the sequence's length after this step), max_q the longest portion.
 // Positions ascend by one along each item's rows.
 void window_attn_mfma(Tensor q, Tensor k_cache, Tensor v_cache, Tensor positions, Tensor cu_q, Tensor k_lens,
                       int64_t max_q, Tensor block_tables, c10::optional<Tensor> bias, int64_t window, Tensor out, int64_t H,
-                      int64_t G) {
+                      int64_t G, c10::optional<Tensor> sink) {
   want(q, torch::kFloat32, "window_attn_mfma q");
   want(positions, torch::kInt32, "window_attn_mfma positions");
   want(block_tables, torch::kInt32, "window_attn_mfma block_tables");
@@ -271,14 +281,16 @@ void window_attn_mfma(Tensor q, Tensor k_cache, Tensor v_cache, Tensor positions
   done(r32_window_attn_mfma(q.data_ptr<float>(), k_cache.data_ptr(), v_cache.data_ptr(), (long long)k_cache.stride(0),
                             (long long)v_cache.stride(0), BS, positions.data_ptr<int>(), cu_q.data_ptr<int>(),
                             k_lens.data_ptr<int>(), items, (int)max_q, block_tables.data_ptr<int>(),
-                            (int)block_tables.size(1), bias.has_value() ? bias->data_ptr<float>() : nullptr, (int)window,
-                            out.data_ptr(), ldo, (int)H, (int)G, D, Dv, stream()), "window_attn_mfma");
+                            (int)block_tables.size(1), bias.has_value() ? bias->data_ptr<float>() : nullptr,
+                            sink_ptr(sink, H, "window_attn_mfma"), (int)window, out.data_ptr(), ldo, (int)H, (int)G, D, Dv,
+                            stream()), "window_attn_mfma");
 }
 
 // One new token per sequence on the matrix cores (bf16 caches): row b reads table row b, its key range ends at
 // positions[b].  max_keys: a host-side upper bound of the keys a row sees (min(window, longest context)).
 void window_attn_decode(Tensor q, Tensor k_cache, Tensor v_cache, Tensor positions, Tensor block_tables,
-                        c10::optional<Tensor> bias, int64_t window, int64_t max_keys, Tensor out, int64_t H, int64_t G) {
+                        c10::optional<Tensor> bias, int64_t window, int64_t max_keys, Tensor out, int64_t H, int64_t G,
+                        c10::optional<Tensor> sink) {
   want(q, torch::kFloat32, "window_attn_decode q");
   want(positions, torch::kInt32, "window_attn_decode positions");
   want(block_tables, torch::kInt32, "window_attn_decode block_tables");
@@ -291,7 +303,7 @@ void window_attn_decode(Tensor q, Tensor k_cache, Tensor v_cache, Tensor positio
   cache_layout(k_cache, v_cache, NB, BS, nk, nv, "window_attn_decode");
   TORCH_CHECK(G > 0 && H > 0 && H % G == 0 && nk % G == 0 && nv % G == 0, "window_attn_decode: head counts");
   const int D = nk / (int)G, Dv = nv / (int)G;
-  TORCH_CHECK(r32_window_attn_mfma_ok(D, Dv), "window_attn_decode: sizes not built");
+  TORCH_CHECK(r32_window_attn_decode_ok(D, Dv), "window_attn_decode: sizes not built");
   const int ldo = row_stride(out, "window_attn_decode out");
   TORCH_CHECK(k_cache.stride(0) % 8 == 0 && v_cache.stride(0) % 8 == 0 && ((uintptr_t)k_cache.data_ptr() & 15) == 0 &&
                   ((uintptr_t)v_cache.data_ptr() & 15) == 0, "window_attn_decode: cache alignment");
@@ -303,8 +315,8 @@ void window_attn_decode(Tensor q, Tensor k_cache, Tensor v_cache, Tensor positio
   float* po = part.data_ptr<float>();
   done(r32_window_attn_decode(q.data_ptr<float>(), k_cache.data_ptr(), v_cache.data_ptr(), (long long)k_cache.stride(0),
                               (long long)v_cache.stride(0), BS, positions.data_ptr<int>(), block_tables.data_ptr<int>(),
-                              (int)block_tables.size(1), bias.has_value() ? bias->data_ptr<float>() : nullptr, (int)window, po,
-                              po + (int64_t)B * H * S * Dv, S,
+                              (int)block_tables.size(1), bias.has_value() ? bias->data_ptr<float>() : nullptr,
+                              sink_ptr(sink, H, "window_attn_decode"), (int)window, po, po + (int64_t)B * H * S * Dv, S,
                               (int)max_keys, out.data_ptr(), ldo, B, (int)H, (int)G, D, Dv, stream()), "window_attn_decode");
 }
 
@@ -718,6 +730,7 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
   m.def("window_attn", &window_attn);
   m.def("window_attn_mfma", &window_attn_mfma);
   m.def("window_attn_mfma_ok", &window_attn_mfma_ok);
+  m.def("window_attn_decode_ok", &window_attn_decode_ok);
   m.def("window_attn_decode", &window_attn_decode);
   m.def("conv_hist", &conv_hist);
   m.def("conv_hist_update", &conv_hist_update);

@@ -2,6 +2,8 @@
 //
 //   score(i, j) = q_i . k_j - r1_h * ln(1 + r2_h * (i - j))        for 0 <= i - j < window
 //   out_i       = softmax_j(score) . v_j
+// With a sink (fp32 per head) the softmax's denominator also holds exp(sink_h): a share of the weight that belongs
+// to no key and adds no value.
 // q arrives in fp32 already multiplied by the head's softmax scale; K rows have D elements, V rows Dv (any sizes,
 // D != Dv allowed), G key/value heads serve H query heads (head h reads group h / (H / G)).  Scores, the softmax
 // and the weighted sum are fp32 whatever the cache's element type (bf16 or fp32).
@@ -211,6 +213,7 @@ struct WAttnMfmaParams {
   const int* block_tables;
   int bt_width;
   const float* bias;  // [H, window], or null: no distance bias
+  const float* sink;  // [H], or null: exp(sink_h) joins the softmax denominator of head h (no key, no value)
   int window;
   bf16_t* out;
   int ldo, H, G;
@@ -426,10 +429,16 @@ __global__ void __launch_bounds__(256) window_attn_mfma_kernel(const WAttnMfmaPa
     __syncthreads();
   }
   if (!wave_live) return;
+  float a_fin = 1.0f;
+  if (p.sink) {  // the sink's share: one more term of the denominator, nothing added to O
+    const float sk = p.sink[h] * kLog2e, mf = fmaxf(m, sk);
+    a_fin = __builtin_amdgcn_exp2f(m - mf);
+    l = l * a_fin + __builtin_amdgcn_exp2f(sk - mf);
+  }
 #pragma unroll
   for (int r = 0; r < 4; ++r) {
     const float lr = __shfl(l, 4 * g4 + r, 64);
-    const float inv = lr > 0.f ? 1.0f / lr : 0.f;
+    const float inv = (lr > 0.f ? 1.0f / lr : 0.f) * __shfl(a_fin, 4 * g4 + r, 64);
     const int row = 16 * w + 4 * g4 + r;
     if (row < nrows) {
       bf16_t* orow = p.out + (size_t)(row0 + row) * p.ldo + (size_t)h * DV;
@@ -452,14 +461,14 @@ int launch_mfma_nv(const WAttnMfmaParams& p, int nv, dim3 grid, size_t shm, hipS
 
 // Whether the matrix-core kernel takes these sizes (bf16 cache only).
 extern "C" int r32_window_attn_mfma_ok(int D, int Dv) {
-  return (D == 32 || D == 64 || D == 128) && (Dv == 32 || Dv == 64 || Dv == 128);
+  return (D == 32 || D == 64 || D == 128 || D == 192) && (Dv == 32 || Dv == 64 || Dv == 128);
 }
 
 extern "C" int r32_window_attn_mfma(const float* q, const void* k_cache, const void* v_cache, long long kb_stride,
                                     long long vb_stride, int block_size, const int* positions, const int* cu_q,
                                     const int* k_lens, int n_items, int max_q, const int* block_tables, int bt_width,
-                                    const float* bias, int window, void* out, int ldo, int H, int G, int D, int Dv,
-                                    hipStream_t s) {
+                                    const float* bias, const float* sink, int window, void* out, int ldo, int H, int G,
+                                    int D, int Dv, hipStream_t s) {
   if (n_items <= 0 || max_q <= 0) return 0;
   if (!r32_window_attn_mfma_ok(D, Dv) || H % G != 0 || (block_size & (block_size - 1)) != 0) return -1;
   WAttnMfmaParams p;
@@ -469,7 +478,7 @@ extern "C" int r32_window_attn_mfma(const float* q, const void* k_cache, const v
   for (int b = 0; b < 20; ++b)
     if ((1 << b) == block_size) p.bs_shift = b;
   p.cu_q = cu_q; p.k_lens = k_lens; p.tiles_per_item = (max_q + 63) / 64; p.block_tables = block_tables;
-  p.bt_width = bt_width; p.bias = bias; p.window = window; p.out = (bf16_t*)out; p.ldo = ldo; p.H = H; p.G = G;
+  p.bt_width = bt_width; p.bias = bias; p.sink = sink; p.window = window; p.out = (bf16_t*)out; p.ldo = ldo; p.H = H; p.G = G;
   const dim3 grid(n_items * p.tiles_per_item, H);
   // a workgroup's keys span at most window + 63 positions (from a 32-aligned start: + 31) and never more than the table
   long long span = (long long)window + 63 + 31;
@@ -480,6 +489,7 @@ extern "C" int r32_window_attn_mfma(const float* q, const void* k_cache, const v
     case 1: return launch_mfma_nv<1>(p, Dv / 16, grid, shm, s);
     case 2: return launch_mfma_nv<2>(p, Dv / 16, grid, shm, s);
     case 4: return launch_mfma_nv<4>(p, Dv / 16, grid, shm, s);
+    case 6: return launch_mfma_nv<6>(p, Dv / 16, grid, shm, s);
   }
   return -1;
 }

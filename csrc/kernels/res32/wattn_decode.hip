@@ -9,7 +9,11 @@ LWC_DEVICE float4v mfma16(const short8& a, const short8& b, const float4v& c) {
   return __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, a), __builtin_bit_cast(bf16x8_t, b), c, 0, 0, 0);
 }
 
-extern "C" int r32_window_attn_mfma_ok(int D, int Dv);
+// Sizes the decode kernel is built for.
+extern "C" int r32_window_attn_decode_ok(int D, int Dv) {
+  const bool small = (D == 32 || D == 64 || D == 128) && (Dv == 32 || Dv == 64 || Dv == 128);
+  return small || (D == 576 && Dv == 512);
+}
 
 // ---------------------------------------------------------------------------------------------------------
 // window_attn_decode_kernel: one new token per sequence on the matrix cores (bf16 cache), split over the keys.
@@ -163,14 +167,17 @@ __global__ void __launch_bounds__(64) window_attn_decode_kernel(const WAttnDecod
 }
 
 // out[b, h, :] = sum_s exp(m_s - M) o_s / sum_s exp(m_s - M) l_s  (splits that saw no key have l = 0)
+// sink (or null): exp(sink_h) joins the denominator.
 __global__ void window_attn_reduce_kernel(const float* __restrict__ part_o, const float* __restrict__ part_ml,
-                                          bf16_t* __restrict__ out, int ldo, int H, int S, int Dv) {
+                                          const float* __restrict__ sink, bf16_t* __restrict__ out, int ldo, int H, int S,
+                                          int Dv) {
   const int b = blockIdx.x, h = blockIdx.y;
   const float* ml = part_ml + ((size_t)b * H + h) * S * 2;
   float M = -1e30f;
   for (int s = 0; s < S; ++s)
     if (ml[2 * s + 1] > 0.f) M = fmaxf(M, ml[2 * s]);
-  float L = 0.f;
+  if (sink) M = fmaxf(M, sink[h]);
+  float L = sink ? expf(sink[h] - M) : 0.f;
   for (int s = 0; s < S; ++s)
     if (ml[2 * s + 1] > 0.f) L += expf(ml[2 * s] - M) * ml[2 * s + 1];
   const float inv = L > 0.f ? 1.0f / L : 0.f;
@@ -209,10 +216,11 @@ extern "C" int r32_window_attn_decode_splits(int B, int G, int Hg, int max_keys)
 // the keys any row sees (min(window, longest context)), known on the host.
 extern "C" int r32_window_attn_decode(const float* q, const void* k_cache, const void* v_cache, long long kb_stride,
                                       long long vb_stride, int block_size, const int* positions, const int* block_tables,
-                                      int bt_width, const float* bias, int window, float* part_o, float* part_ml, int S,
-                                      int max_keys, void* out, int ldo, int B, int H, int G, int D, int Dv, hipStream_t s) {
+                                      int bt_width, const float* bias, const float* sink, int window, float* part_o,
+                                      float* part_ml, int S, int max_keys, void* out, int ldo, int B, int H, int G, int D,
+                                      int Dv, hipStream_t s) {
   if (B <= 0) return 0;
-  if (!r32_window_attn_mfma_ok(D, Dv) || H % G != 0 || S < 1 || (block_size & (block_size - 1)) != 0) return -1;
+  if (!r32_window_attn_decode_ok(D, Dv) || H % G != 0 || S < 1 || (block_size & (block_size - 1)) != 0) return -1;
   WAttnDecodeParams p;
   p.q = q; p.k_cache = (const bf16_t*)k_cache; p.v_cache = (const bf16_t*)v_cache; p.kb_stride = kb_stride;
   p.vb_stride = vb_stride; p.block_size = block_size; p.positions = positions; p.block_tables = block_tables;
@@ -226,12 +234,17 @@ extern "C" int r32_window_attn_decode(const float* q, const void* k_cache, const
   const int Hg = H / G;
   const dim3 grid(B, G * ((Hg + 15) / 16), S);
   int rc = -1;
-  switch (D / 32) {
-    case 1: rc = launch_decode_nv<1>(p, Dv / 16, grid, s); break;
-    case 2: rc = launch_decode_nv<2>(p, Dv / 16, grid, s); break;
-    case 4: rc = launch_decode_nv<4>(p, Dv / 16, grid, s); break;
+  if (D == 576 && Dv == 512) {  // one wide row for all heads: a low-rank attention's cached latent + rotated part
+    window_attn_decode_kernel<18, 32><<<grid, 64, 0, s>>>(p);
+    rc = (int)hipGetLastError();
+  } else {
+    switch (D / 32) {
+      case 1: rc = launch_decode_nv<1>(p, Dv / 16, grid, s); break;
+      case 2: rc = launch_decode_nv<2>(p, Dv / 16, grid, s); break;
+      case 4: rc = launch_decode_nv<4>(p, Dv / 16, grid, s); break;
+    }
   }
   if (rc != 0) return rc;
-  window_attn_reduce_kernel<<<dim3(B, H), 64, 0, s>>>(part_o, part_ml, (bf16_t*)out, ldo, H, S, Dv);
+  window_attn_reduce_kernel<<<dim3(B, H), 64, 0, s>>>(part_o, part_ml, sink, (bf16_t*)out, ldo, H, S, Dv);
   return (int)hipGetLastError();
 }

@@ -53,6 +53,24 @@ def _up(n: int, m: int) -> int:
     return -(-n // m) * m
 
 
+def _core_size(n: int) -> int:
+    """The next head size the matrix-core attention kernels are built for (beyond 128: a multiple of 8)."""
+    for c in (32, 64, 128):
+        if n <= c:
+            return c
+    return _up(n, 8)
+
+
+@dataclass
+class StepAttention:
+    """How a step's rows reach the paged cache: ``n_dec`` decode rows (row b reads ``dec_tables[b]``), then prompt
+    portions described by ``chunk`` (block tables, row offsets, key counts; host copies of the counts in "lens")."""
+    n_dec: int
+    dec_tables: Optional[torch.Tensor]
+    chunk: Optional[dict]
+    scratch: Dict[object, object] = field(default_factory=dict)   # per-step data shared by the layer runs
+
+
 @dataclass
 class LimatarLayer:
     norm1: torch.Tensor                  # fp32, 1 + w
@@ -200,6 +218,8 @@ class LimatarModel:
                 x["w_uq"] = t(p + "mix.uq")
                 x["w_uk"] = t(p + "mix.uk").view(m.heads, m.dim, m.kv_rank)                               # [H, D, C]
                 x["w_uv_t"] = t(p + "mix.uv").view(m.heads, m.vdim, m.kv_rank).transpose(1, 2).contiguous()  # [H, C, Dv]
+                if self.expanded_head_sizes(m) is not None:
+                    x["w_ukv"] = torch.cat([t(p + "mix.uk"), t(p + "mix.uv")], 0).contiguous()
             else:
                 w_in = torch.cat([t(p + "mix.q"), t(p + "mix.k"), t(p + "mix.v"), t(p + "mix.g")], 0).contiguous()
                 x["decay"] = torch.tensor(m.decay, dtype=torch.float32, device=dev)
@@ -257,11 +277,27 @@ class LimatarModel:
                 gemm_plan.tune(torch.randn(M, w.shape[1], device=self.device).to(self.dtype), w, ws=self.g8_ws, bucket=bucket)
 
     # ------------------------------------------------------------------ cache and state
-    @staticmethod
-    def latent_row_sizes(m) -> tuple:
+    def latent_row_sizes(self, m) -> tuple:
         """(key row, value row) sizes of a low-rank attention layer's cached token: [latent | rotated part] and the
-        latent, each padded with zeros to a multiple of 8 entries (16-byte rows)."""
-        return _up(m.kv_rank + m.rot_dim, 8), _up(m.kv_rank, 8)
+        latent, padded with zeros.  bf16: up to the next size the matrix-core attention kernels are built for (32, 64,
+        128; one wide row of 576 / 512 for latents above 288 entries), else to a multiple of 8 (16-byte rows)."""
+        nk, nv = m.kv_rank + m.rot_dim, m.kv_rank
+        if self.dtype == torch.bfloat16:
+            if nk <= 128:
+                return _core_size(nk), _core_size(nv)
+            if 288 < nk <= 576 and nv <= 512:
+                return 576, 512
+        return _up(nk, 8), _up(nv, 8)
+
+    def expanded_head_sizes(self, m) -> Optional[tuple]:
+        """(key, value) sizes per head of the up-projected keys [unrotated | rotated part] and values that prompt
+        portions attend over when the cached rows themselves are too wide for the portion kernel; None: not used."""
+        K = res32.kernels()
+        if self.dtype != torch.bfloat16 or K.window_attn_mfma_ok(*self.latent_row_sizes(m)):
+            return None
+        dk = _core_size(m.dim + m.rot_dim) if m.dim + m.rot_dim <= 128 else _up(m.dim + m.rot_dim, 64)
+        dv = _core_size(m.vdim)
+        return (dk, dv) if K.window_attn_mfma_ok(dk, dv) else None
 
     def _layer_dims(self):
         return [self.latent_row_sizes(self.cfg.layer_specs[self.runs[ri]].mixer) for ri in sorted(self.cache_index)]
@@ -297,7 +333,7 @@ class LimatarModel:
             return torch.bmm(a, b, out_dtype=torch.float32)
         return torch.bmm(a.float(), b.float())
 
-    def _latent_mixer(self, h, L: LimatarLayer, m, ri: int, positions, slots, cache, attend) -> torch.Tensor:
+    def _latent_mixer(self, h, L: LimatarLayer, m, ri: int, positions, slots, cache, plan: StepAttention) -> torch.Tensor:
         x, T, dt = L.extra, h.shape[0], self.dtype
         C, R, D, H = m.kv_rank, m.rot_dim, m.dim, m.heads
         ci = self.cache_index[ri]
@@ -306,14 +342,81 @@ class LimatarModel:
         cq = res32.latent_kv_write(proj, m.q_rank, C, R, x["dq_norm"], x["dkv_norm"], x["freq"], x["rot_mult"], positions,
                                    slots, cache.k[ci], cache.v[ci], self.cfg.norm_eps)
         q = self._linear(cq, x["w_uq"])                                            # [T, H (D + R)]
-        qn = self._bmm32(q.view(T, H, D + R)[:, :, :D].transpose(0, 1), x["w_uk"])  # [H, T, C]: keys' up-projection on q
-        qf = res32.latent_q_rows(q, D, R, qn, x["freq"], x["rot_mult"], m.scale, positions, H, Dk)
-        oc = torch.empty(T, H * Cv, dtype=dt, device=self.device)
-        attend(qf.view(T, H * Dk), ri, oc)
-        o = torch.bmm(oc.view(T, H, Cv)[:, :, :C].transpose(0, 1), x["w_uv_t"])    # [H, T, Dv]
-        a = o.transpose(0, 1).reshape(T, H * m.vdim)
+        n_dec = plan.n_dec
+        wide = T > n_dec and self.expanded_head_sizes(m) is not None and cache.block_size & (cache.block_size - 1) == 0
+        n_abs = n_dec if wide else T   # rows that attend over the cached latent rows themselves
+        a = torch.empty(T, H * m.vdim, dtype=dt, device=self.device)
+        z, kc, vc = self._no_bias(H), cache.k[ci], cache.v[ci]
+        if n_abs:
+            qa, pa = q[:n_abs], positions[:n_abs]
+            qn = self._bmm32(qa.view(n_abs, H, D + R)[:, :, :D].transpose(0, 1), x["w_uk"])  # [H, n, C]: keys' up-projection on q
+            qf = res32.latent_q_rows(qa, D, R, qn, x["freq"], x["rot_mult"], m.scale, pa, H, Dk).view(n_abs, H * Dk)
+            oc = torch.empty(n_abs, H * Cv, dtype=dt, device=self.device)
+            if n_dec:
+                res32.window_attn(qf[:n_dec], kc, vc, pa[:n_dec], plan.dec_tables, z, z, UNBOUNDED, oc[:n_dec], H, 1,
+                                  cores=True, sink=x["sink"])
+            if n_abs > n_dec:
+                ch = plan.chunk
+                res32.window_attn(qf[n_dec:], kc, vc, pa[n_dec:], ch["block_tables"], z, z, UNBOUNDED, oc[n_dec:], H, 1,
+                                  cu_q=ch["cu_q"], k_lens=ch.get("k_lens"), max_q=int(ch.get("max_q", 0)), cores=True,
+                                  sink=x["sink"])
+            o = torch.bmm(oc.view(n_abs, H, Cv)[:, :, :C].transpose(0, 1), x["w_uv_t"])      # [H, n, Dv]
+            a[:n_abs] = o.transpose(0, 1).reshape(n_abs, H * m.vdim)
+        if wide:
+            a[n_dec:] = self._expanded_attention(q[n_dec:], positions[n_dec:], L, m, kc, cache.block_size, plan)
         res32.gate_mul(a, proj[:, m.q_rank + C + R:], "sigmoid")
         return a
+
+    def _context_rows(self, plan: StepAttention, bs: int) -> dict:
+        """For the prompt portions of a step: where every token of their sequences (the keys they may see) lies in the
+        paged cache, and a dense page numbering of those tokens, sequence after sequence (built once per step)."""
+        ctx = plan.scratch.get("ctx")
+        if ctx is None:
+            ch = plan.chunk
+            k_lens = np.asarray(ch["lens"][1], dtype=np.int64)
+            pages = -(-k_lens // bs)
+            first = np.concatenate([[0], np.cumsum(pages)])
+            item = np.repeat(np.arange(len(k_lens)), k_lens)
+            pos = np.concatenate([np.arange(n) for n in k_lens]) if len(k_lens) else np.zeros(0, np.int64)
+            dev = self.device
+            item_d, pos_d = torch.from_numpy(item).to(dev), torch.from_numpy(pos).to(dev)
+            blk = ch["block_tables"][item_d, pos_d // bs].long()
+            tables = np.zeros((len(k_lens), max(1, int(pages.max()))), np.int32)
+            for i, n in enumerate(pages):
+                tables[i, :n] = first[i] + np.arange(n)
+            ctx = plan.scratch["ctx"] = {"blk": blk, "off": pos_d % bs, "slots": torch.from_numpy(first[item] * bs + pos).to(dev),
+                                         "tables": torch.from_numpy(tables).to(dev), "pages": int(first[-1])}
+        return ctx
+
+    def _expanded_attention(self, q, positions, L: LimatarLayer, m, k_rows, bs: int, plan: StepAttention) -> torch.Tensor:
+        """Prompt portions over keys and values up-projected from the cached latents of their sequences: per head the
+        key [W_uk c | rotated part] and the value W_uv c, laid out as pages of their own for the portion kernel."""
+        x, Tq = L.extra, q.shape[0]
+        C, R, D, H, Dv = m.kv_rank, m.rot_dim, m.dim, m.heads, m.vdim
+        dk, dv = self.expanded_head_sizes(m)
+        ctx = self._context_rows(plan, bs)
+        rows = k_rows[ctx["blk"], ctx["off"]]                                      # [N, row]: latent | rotated part
+        N = rows.shape[0]
+        kv = F.linear(rows[:, :C], x["w_ukv"])                                     # [N, H D + H Dv]
+        kexp = torch.zeros(N, H, dk, dtype=self.dtype, device=self.device)
+        kexp[:, :, :D] = kv[:, :H * D].view(N, H, D)
+        kexp[:, :, D:D + R] = rows[:, None, C:C + R]
+        vexp = kv[:, H * D:]
+        if dv != Dv:
+            vexp = torch.zeros(N, H, dv, dtype=self.dtype, device=self.device)
+            vexp[:, :, :Dv] = kv[:, H * D:].view(N, H, Dv)
+        key = ("pages", H * dk, H * dv)
+        tmp = plan.scratch.get(key)
+        if tmp is None:
+            tmp = plan.scratch[key] = PagedLayerCache([(H * dk, H * dv)], ctx["pages"], bs, self.device, self.dtype)
+        tmp.set_rows(0, ctx["slots"], kexp.view(N, H * dk), vexp.reshape(N, H * dv))
+        qn = q.view(Tq, H, D + R)[:, :, :D].permute(1, 0, 2).float().contiguous()   # [H, Tq, D]
+        qf = res32.latent_q_rows(q, D, R, qn, x["freq"], x["rot_mult"], m.scale, positions, H, dk)
+        out = torch.empty(Tq, H * dv, dtype=self.dtype, device=self.device)
+        ch, z = plan.chunk, self._no_bias(H)
+        res32.window_attn(qf.view(Tq, H * dk), tmp.k[0], tmp.v[0], positions, ctx["tables"], z, z, UNBOUNDED, out, H, H,
+                          cu_q=ch["cu_q"], k_lens=ch["k_lens"], max_q=int(ch["max_q"]), cores=True, sink=x["sink"])
+        return out if dv == Dv else out.view(Tq, H, dv)[:, :, :Dv].reshape(Tq, H * Dv)
 
     def _retention_mixer(self, h, L: LimatarLayer, m, ri: int, state, items) -> torch.Tensor:
         x, T = L.extra, h.shape[0]
@@ -348,8 +451,8 @@ class LimatarModel:
         return res32.moe_combine(Y, inv, w, h2, add=shared)
 
     def _forward(self, tokens, positions, slots, cache: PagedLayerCache, state: RecurrentStatePool,
-                 items: res32.StepItems, attend, keep: Optional[torch.Tensor] = None) -> torch.Tensor:
-        """Every layer run over the step's rows; ``attend(q, run, out)`` runs the attention of a run into ``out``.
+                 items: res32.StepItems, plan: StepAttention, keep: Optional[torch.Tensor] = None) -> torch.Tensor:
+        """Every layer run over the step's rows; ``plan`` says how the rows reach the paged cache.
         Returns the fp32 stream that the output norm reads, [T, d].
 
         ``keep`` (int64 rows): only these rows' final states are wanted (a prompt's last token).  The LAST run then
@@ -361,7 +464,7 @@ class LimatarModel:
             S, L = cfg.layer_specs[li], self.layers[li]
             h = res32.rmsnorm_rows(x, L.norm1, eps, dt)
             if S.type == "latent_attention":
-                a = self._latent_mixer(h, L, S.mixer, ri, positions, slots, cache, attend)
+                a = self._latent_mixer(h, L, S.mixer, ri, positions, slots, cache, plan)
             else:
                 a = self._retention_mixer(h, L, S.mixer, ri, state, items)
             if keep is not None and ri + 1 == len(self.runs):   # from here on only the kept rows
@@ -392,17 +495,6 @@ class LimatarModel:
             z = self._zeros_h[H] = torch.zeros(H, dtype=torch.float32, device=self.device)
         return z
 
-    def _attend(self, cache, positions, tables, cu_q=None, k_lens=None, max_q=0):
-        def run(q, ri, out, rows=slice(None)):
-            L = self.layers[self.runs[ri]]
-            m = self.cfg.layer_specs[self.runs[ri]].mixer
-            ci = self.cache_index[ri]
-            z = self._no_bias(m.heads)
-            res32.window_attn(q[rows], cache.k[ci], cache.v[ci], positions[rows], tables, z, z, UNBOUNDED, out[rows],
-                              m.heads, 1, cu_q=cu_q, k_lens=k_lens, max_q=max_q, bias=None, cores=True,
-                              sink=L.extra["sink"])
-        return run
-
     def decode(self, tokens: torch.Tensor, positions: torch.Tensor, slots: torch.Tensor, block_tables: torch.Tensor,
                ctx_lens: torch.Tensor, cache: PagedLayerCache, num_splits: int = 1, cascade_tiles=None,
                float_logits: bool = False, state: Optional[RecurrentStatePool] = None,
@@ -412,7 +504,7 @@ class LimatarModel:
         if state is None or state_slots is None:
             raise RuntimeError("Limatar: a decode step needs the recurrent-state pool and the rows' slots")
         items = res32.StepItems.rows(state_slots, positions)
-        x = self._forward(tokens, positions, slots, cache, state, items, self._attend(cache, positions, block_tables))
+        x = self._forward(tokens, positions, slots, cache, state, items, StepAttention(tokens.shape[0], block_tables, None))
         return self._logits(x, None, float_logits)
 
     def forward_mixed(self, tokens: torch.Tensor, positions: torch.Tensor, slots: torch.Tensor, cache: PagedLayerCache,
@@ -434,18 +526,9 @@ class LimatarModel:
         dev = self.device
         items = res32.StepItems(torch.from_numpy(row_item.astype(np.int32)).to(dev), torch.from_numpy(cu.astype(np.int32)).to(dev),
                                 state_slots, positions)
-        dec_run = self._attend(cache, positions, dec["block_tables"]) if n_dec else None
-        chk_run = (self._attend(cache, positions, chunk["block_tables"], cu_q=chunk["cu_q"], k_lens=chunk.get("k_lens"),
-                                max_q=int(chunk.get("max_q", 0))) if T > n_dec else None)
-
-        def attend(q, ri, out):
-            if dec_run is not None:
-                dec_run(q, ri, out, slice(0, n_dec))
-            if chk_run is not None:
-                chk_run(q, ri, out, slice(n_dec, T))
-
+        plan = StepAttention(n_dec, dec["block_tables"] if n_dec else None, chunk if T > n_dec else None)
         keep = logit_rows if n_dec == 0 and self.on_layer is None and 4 * logit_rows.numel() <= T else None
-        x = self._forward(tokens, positions, slots, cache, state, items, attend, keep=keep)
+        x = self._forward(tokens, positions, slots, cache, state, items, plan, keep=keep)
         return self._logits(x, None if keep is not None else logit_rows, float_logits)
 
     def prefill(self, tokens, positions, slots, cu_seqlens, max_seqlen, last_idx, cache, ctx=None):

@@ -115,15 +115,16 @@ def window_attn(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, p
     ``sink`` (fp32 [H]): exp(sink_h) joins head h's softmax denominator; it has no key and no value."""
     K = kernels()
     bs = k_cache.shape[1]
-    cores = ((bias is not None or bool(cores)) and sink is None and k_cache.dtype == torch.bfloat16 and bs & (bs - 1) == 0
-             and K.window_attn_mfma_ok(k_cache.shape[2] // G, v_cache.shape[2] // G))
-    if cores and cu_q is None and positions.numel() > 0:
+    D, Dv = k_cache.shape[2] // G, v_cache.shape[2] // G
+    cores = (bias is not None or bool(cores)) and k_cache.dtype == torch.bfloat16 and bs & (bs - 1) == 0
+    if cores and cu_q is None and positions.numel() > 0 and K.window_attn_decode_ok(D, Dv):
         max_keys = min(int(window), block_tables.shape[1] * k_cache.shape[1])
-        K.window_attn_decode(q, k_cache, v_cache, positions, block_tables, bias, int(window), max_keys, out, int(H), int(G))
+        K.window_attn_decode(q, k_cache, v_cache, positions, block_tables, bias, int(window), max_keys, out, int(H), int(G),
+                             sink)
         return out
-    if cores and cu_q is not None and k_lens is not None and max_q > 0:
+    if cores and cu_q is not None and k_lens is not None and max_q > 0 and K.window_attn_mfma_ok(D, Dv):
         K.window_attn_mfma(q, k_cache, v_cache, positions, cu_q, k_lens, int(max_q), block_tables, bias, int(window), out,
-                           int(H), int(G))
+                           int(H), int(G), sink)
         return out
     K.window_attn(q, k_cache, v_cache, positions, cu_q, block_tables, r1, r2, int(window), out, int(H), int(G), sink)
     return out

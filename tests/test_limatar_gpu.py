@@ -100,10 +100,13 @@ def _paged(n_tokens, bs, nk, nv, dtype, gpu, seed=0):
 
 
 @pytest.mark.parametrize("dtype,tol", [(torch.float32, 2e-5), (torch.bfloat16, 2e-2)])
-@pytest.mark.parametrize("H,D,Dv", [(3, 40, 24), (8, 112, 96), (2, 328, 320), (1, 8, 8)])
+@pytest.mark.parametrize("H,D,Dv", [(3, 40, 24), (8, 112, 96), (2, 328, 320), (1, 8, 8), (4, 128, 128), (5, 64, 32), (3, 192, 128),
+                                    (17, 576, 512)])
 def test_softmax_with_sinks_over_one_shared_row(gpu, dtype, tol, H, D, Dv):
     """All heads read ONE cached row per token (G = 1); exp(sink_h) joins the denominator.  Decode rows and a prompt
-    portion behind a cached head, sinks from far below to far above the scores."""
+    portion behind a cached head, sinks from far below to far above the scores.  In bf16 the sizes the matrix-core
+    kernels are built for run there (decode rows split over the keys; 17 heads: two head chunks), the rest and fp32 on
+    the general kernel."""
     from llm_weighted_consensus_amd.ops import res32
 
     g = torch.Generator().manual_seed(D)
@@ -122,13 +125,13 @@ def test_softmax_with_sinks_over_one_shared_row(gpu, dtype, tol, H, D, Dv):
     rows = [0, 1, 15, 16, 17, 82]  # decode rows: every row its own item
     out = torch.empty(len(rows), H * Dv, dtype=dtype, device=gpu)
     res32.window_attn(q[rows].reshape(len(rows), -1).to(gpu), cache.k[0], cache.v[0], torch.tensor(rows, dtype=torch.int32, device=gpu),
-                      tab.expand(len(rows), -1).contiguous(), z, z, 1 << 30, out, H, 1, sink=sink.to(gpu))
+                      tab.expand(len(rows), -1).contiguous(), z, z, 1 << 30, out, H, 1, sink=sink.to(gpu), cores=True)
     assert (out.cpu().double().view(len(rows), H, Dv) - ref[rows]).abs().max() < tol * 4
     a = 30  # a portion of rows a .. n-1 behind a cached head
     out = torch.empty(n - a, H * Dv, dtype=dtype, device=gpu)
     res32.window_attn(q[a:].reshape(n - a, -1).to(gpu), cache.k[0], cache.v[0], torch.arange(a, n, dtype=torch.int32, device=gpu), tab, z, z,
                       1 << 30, out, H, 1, cu_q=torch.tensor([0, n - a], dtype=torch.int32, device=gpu),
-                      k_lens=torch.tensor([n], dtype=torch.int32, device=gpu), max_q=n - a, sink=sink.to(gpu))
+                      k_lens=torch.tensor([n], dtype=torch.int32, device=gpu), max_q=n - a, sink=sink.to(gpu), cores=True)
     assert (out.cpu().double().view(n - a, H, Dv) - ref[a:]).abs().max() < tol * 4
     if H > 1:  # the lowest sink changes nothing, the highest takes most of the weight
         w = O.sink_softmax(s, sink.double())[:, -1].sum(-1)
@@ -136,13 +139,13 @@ def test_softmax_with_sinks_over_one_shared_row(gpu, dtype, tol, H, D, Dv):
 
 
 @pytest.mark.parametrize("decode", [False, True])
-@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
-def test_far_key_and_page_borders_stand_out(gpu, decode, dtype):
+@pytest.mark.parametrize("dtype,D,Dv", [(torch.float32, 24, 16), (torch.bfloat16, 24, 16), (torch.bfloat16, 128, 64)])
+def test_far_key_and_page_borders_stand_out(gpu, decode, dtype, D, Dv):
     """One key made to stand out (its row parallel to the query, scaled up) at the first token, at both sides of page
     borders and hundreds of tokens back over shuffled pages: the result is that key's value row, less the sink's share."""
     from llm_weighted_consensus_amd.ops import res32
 
-    H, D, Dv, n, bs = 2, 24, 16, 300, 16
+    H, n, bs = 2, 300, 16
     g = torch.Generator().manual_seed(5)
     z = torch.zeros(H, device=gpu)
     sink = torch.tensor([-50.0, 2.0])
@@ -158,7 +161,7 @@ def test_far_key_and_page_borders_stand_out(gpu, decode, dtype):
         kw = {} if decode else dict(cu_q=torch.tensor([0, 1], dtype=torch.int32, device=gpu),
                                     k_lens=torch.tensor([n], dtype=torch.int32, device=gpu), max_q=1)
         res32.window_attn(q, cache.k[0], cache.v[0], torch.tensor([n - 1], dtype=torch.int32, device=gpu), table[None].to(gpu), z, z,
-                          1 << 30, out, H, 1, sink=sink.to(gpu), **kw)
+                          1 << 30, out, H, 1, sink=sink.to(gpu), cores=True, **kw)
         got = out.cpu().double().view(H, Dv)
         want = V[target].to(dtype).double()
         assert (got[0] - want).abs().max() < 2e-2, target                       # no sink to speak of
@@ -306,6 +309,13 @@ def _configs():
         "grouped": dict(width=256, vocab=200, loop=None, layers=[
             O.retention_layer(2, 32, 32, O.moe(4, 2, 1024, shared=64)), O.latent_layer(2, 32, 16, 32, 32, 48, O.dense(64))]),
     }
+    # cached rows too wide for the portion kernel: prompt portions attend over up-projected keys and values (key sizes
+    # 48 + 16 and 100 + 32 -> 192, values padded 40 -> 64), decode rows over the latent rows on the general kernel
+    out["wide"] = dict(width=64, vocab=200, loop=(0, 1, 2), layers=[
+        O.latent_layer(3, 48, 16, 32, 40, 200, O.dense(64)), O.latent_layer(2, 100, 32, 40, 24, 136, m8, scaling=SCALING)])
+    # a latent wide enough for the 576 / 512 decode kernel (17 heads: two head chunks)
+    out["deep"] = dict(width=64, vocab=200, loop=None, layers=[
+        O.latent_layer(17, 16, 64, 16, 24, 320, O.dense(64)), O.retention_layer(2, 16, 16, None)])
     # the same layers with two passes of the span: bf16 comparisons (rounding differences grow with every pass of the
     # same weights, and a routing choice flipped by rounding changes a whole row)
     out["mixed2"] = {**out["mixed"], "loop": (1, 3, 2)}
@@ -362,7 +372,7 @@ def _err(got, ref, dtype=torch.float32):
 TOL = {torch.float32: 1e-4, torch.bfloat16: 0.5}
 
 
-@pytest.mark.parametrize("name,dtype", [(n, d) for d in (torch.float32, torch.bfloat16) for n in ("mixed", "odd", "recurrent", "attentive")
+@pytest.mark.parametrize("name,dtype", [(n, d) for d in (torch.float32, torch.bfloat16) for n in ("mixed", "odd", "recurrent", "attentive", "wide", "deep")
                                         if (n, d) != ("mixed", torch.bfloat16)] + [("mixed2", torch.bfloat16)])
 def test_whole_prompt_and_layer_runs(gpu, tmp_path, name, dtype):
     """A whole prompt in one step: the stream after every layer RUN (looped layers count each time) and the logits."""
@@ -409,7 +419,8 @@ def test_few_wanted_rows_and_what_they_leave(gpu, tmp_path, name, dtype):
 
 
 @pytest.mark.parametrize("name,dtype", [("mixed", torch.float32), ("odd", torch.float32), ("recurrent", torch.float32),
-                                        ("attentive", torch.bfloat16), ("mixed2", torch.bfloat16)])
+                                        ("attentive", torch.bfloat16), ("mixed2", torch.bfloat16), ("wide", torch.bfloat16),
+                                        ("deep", torch.bfloat16)])
 def test_decode_token_by_token_and_portions(gpu, tmp_path, name, dtype):
     """The same logits whether a prompt comes whole, token by token from the first token on, or in portions of
     changing sizes (down to two tokens; cut inside pages and inside the recurrence kernel's tiles)."""
@@ -431,7 +442,7 @@ def test_decode_token_by_token_and_portions(gpu, tmp_path, name, dtype):
 
 
 @pytest.mark.parametrize("name,dtype", [("mixed", torch.float32), ("mixed2", torch.bfloat16), ("attentive", torch.bfloat16),
-                                        ("odd", torch.float32)])
+                                        ("odd", torch.float32), ("wide", torch.bfloat16), ("deep", torch.bfloat16)])
 def test_unequal_batches_pages_and_slots_used_again(gpu, tmp_path, name, dtype):
     """Up to four live sequences of unequal lengths, portions beside single tokens, one sitting steps out, in a pool
     so small that pages and state slots are freed and taken again; every position equals the sequence run alone."""
@@ -469,7 +480,7 @@ def test_every_pass_of_a_loop_has_its_own_cache_and_state(gpu, tmp_path):
     """Looped layers share weights, not pages or state: with the loop the model differs from the same layers run
     once, and decoding after a prompt (which reads every pass's cache and state) matches the oracle's loop."""
     cfg, W, model, eng = _build(tmp_path, "mixed", torch.float32)
-    assert len(model.cache_index) == 4 and len(model.state_fields()) == 4  # 8 runs of 4 layers
+    assert len(model.runs) == 8 and len(model.cache_index) == 4 and len(model.state_fields()) == 4
     toks = _tokens(40, cfg["vocab"], 12)
     ref = O.forward(cfg, W, toks)
     once = O.forward({**cfg, "loop": None}, W, toks)
