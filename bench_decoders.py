@@ -3,9 +3,12 @@
 
     python bench.py --compare-decoders [--sizes small,8b-layer] [--compare-layers 4]
 
-Designs: ``madipel``, ``llama``, ``merudra``, ``mixtral`` (``--designs merudra,mixtral`` puts Merudra beside the
-closest existing decoder, the routed-experts Mixtral: 8 experts, 2 per token, the same active feed-forward width;
-Merudra's layers alternate attention and gated delta rule mixers and add 2 identity experts).
+Designs: ``madipel``, ``llama``, ``merudra``, ``mixtral``, ``limatar`` (``--designs merudra,mixtral`` puts Merudra
+beside the closest existing decoder, the routed-experts Mixtral: 8 experts, 2 per token, the same active feed-forward
+width; Merudra's layers alternate attention and gated delta rule mixers and add 2 identity experts.
+``--designs limatar,merudra`` puts Limatar beside Merudra, the closest decoder with paged attention AND recurrent
+layers over an fp32 stream: Limatar's layers alternate low-rank attention (latent 512 + 64 rotated entries, sinks) and
+retention, routed experts with a shared expert and the clamped dense unit).
 
 For each size a Madipel model (parallel layers, windowed attention with distance bias, xIELU feed-forward, fp32
 residual) and the closest existing decoder (Llama: sequential layers, causal GQA attention with RoPE, SwiGLU) are
@@ -68,6 +71,32 @@ def _merudra(size: dict, layers: int, device, seed: int, experts: int = 8, top: 
     return MerudraModel(cfg, device=device, seed=seed)
 
 
+def _limatar(size: dict, layers: int, device, seed: int, experts: int = 8, top: int = 2, pattern: str = "lr"):
+    """Low-rank attention and retention layers alternating (``pattern``: l / r per layer, repeated; a / d of the other
+    designs' patterns mean the same), feed-forwards alternating in pairs between routed experts (inner width ffn / top,
+    a shared expert of ffn / 8) and the dense clamped unit of inner width ffn: the same active width everywhere."""
+    from llm_weighted_consensus_amd.models.config import LimatarConfig
+    from llm_weighted_consensus_amd.models.limatar import LimatarModel
+
+    H, D, d = size["heads"], size["head_dim"], size["width"]
+    moe = {"kind": "moe", "expert": {"ff": size["ffn"] // top}, "router": {"experts": experts, "top": top},
+           "shared": {"ff": size["ffn"] // 8}}
+    dense = {"kind": "dense", "ff": size["ffn"], "limit": 7.0}
+    lat = {"heads": H, "dim": D, "rot_dim": D // 2, "vdim": D, "q_rank": 3 * d // 8, "kv_rank": 4 * D, "scale": (D + D // 2) ** -0.5,
+           "rot": {"base": 10000.0, "dims": D // 2, "scaling": {"factor": 4.0, "original": 1024, "fast": 32.0, "slow": 1.0}}}
+    ret = {"heads": H, "dim": D, "vdim": D, "decay": [1.0 - 2.0 ** (-5 - 3 * h / max(H - 1, 1)) for h in range(H)],
+           "rot": {"base": 10000.0, "dims": D}}
+    specs = []
+    for i in range(layers):
+        kind = pattern[i % len(pattern)]
+        mlp = moe if (i // 2 + i) % 2 == 0 else dense
+        specs.append({"type": "latent_attention", "mixer": lat, "mlp": mlp} if kind in "la" else
+                     {"type": "retention", "mixer": ret, "mlp": mlp})
+    cfg = LimatarConfig.from_dict({"architecture": "Limatar", "layers": specs, "norm": {"eps": 1e-6}, "vocab": size["vocab"],
+                                   "width": d}, name="limatar-bench")
+    return LimatarModel(cfg, device=device, seed=seed)
+
+
 def _mixtral(size: dict, layers: int, max_pos: int, device, seed: int, experts: int = 8, top: int = 2):
     from llm_weighted_consensus_amd.models.config import DecoderConfig
     from llm_weighted_consensus_amd.models.mixtral import MixtralModel
@@ -127,7 +156,9 @@ def run(sizes: str = "small,8b-layer", layers: int = 4, prompt_len: int = 2048, 
             if design == "madipel":
                 model = _madipel(size, layers, window, dev, 3)
             elif design == "merudra":
-                model = _merudra(size, layers, dev, 3, pattern=pattern)
+                model = _merudra(size, layers, dev, 3, pattern="".join({"l": "a", "r": "d"}.get(c, c) for c in pattern))
+            elif design == "limatar":
+                model = _limatar(size, layers, dev, 3, pattern=pattern)
             elif design == "mixtral":
                 model = _mixtral(size, layers, prompt_len + gen + 80, dev, 3)
             else:
@@ -141,7 +172,7 @@ def run(sizes: str = "small,8b-layer", layers: int = 4, prompt_len: int = 2048, 
                     **{k: round(v, 3) for k, v in r.items()}, "dtype": "bf16", "data": "synthetic"}
             print(json.dumps(line), flush=True)
             summary.setdefault(name, {})[design] = r
-    for a, b in (("madipel", "llama"), ("merudra", "mixtral"), ("merudra", "madipel")):
+    for a, b in (("madipel", "llama"), ("merudra", "mixtral"), ("merudra", "madipel"), ("limatar", "merudra")):
         out = {}
         for name, d in summary.items():
             if a in d and b in d:

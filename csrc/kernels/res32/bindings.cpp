@@ -22,7 +22,7 @@ int r32_window_attn_mfma(const float*, const void*, const void*, long long, long
                          const int*, int, int, const int*, int, const float*, const float*, int, void*, int, int, int, int, int,
                          hipStream_t);
 int r32_window_attn_decode_ok(int, int);
-int r32_window_attn_decode_splits(int, int, int, int);
+int r32_window_attn_decode_splits(int, int, int, int, int);
 int r32_window_attn_decode(const float*, const void*, const void*, long long, long long, int, const int*, const int*, int,
                            const float*, const float*, int, float*, float*, int, int, void*, int, int, int, int, int, int,
                            hipStream_t);
@@ -38,8 +38,10 @@ int r32_embed_rows(const void*, const int*, float*, int, int, int, int, hipStrea
 int r32_head_norm_kv_write(const void*, int, int, int, const int*, const int*, float*, void*, void*, long long, long long,
                            int, int, int, int, int, int, float, float, float, int, int, hipStream_t);
 int r32_gate_mul(void*, int, const void*, int, int, int, int, int, hipStream_t);
-int r32_gated_norm_residual(float*, const void*, int, const void*, int, const float*, void*, int, int, float, int, int,
-                            hipStream_t);
+int r32_gated_norm_residual(float*, const void*, int, const void*, int, const float*, void*, const float*, int, int, float,
+                            int, int, hipStream_t);
+int r32_latent_expand_write(const void*, int, const void*, int, int, const long long*, void*, void*, long long, long long,
+                            int, int, int, int, int, int, int, int, int, hipStream_t);
 int r32_rmsnorm_rows(const float*, const long long*, const float*, void*, int, int, float, int, hipStream_t);
 int r32_gelu_mul_rows(const void*, int, const void*, int, int, const int*, int, void*, int, int, int, hipStream_t);
 int r32_stack_mix(const float*, long long, const float*, int, float*, long long, hipStream_t);
@@ -310,7 +312,7 @@ void window_attn_decode(Tensor q, Tensor k_cache, Tensor v_cache, Tensor positio
   TORCH_CHECK(block_tables.dim() == 2 && block_tables.size(0) >= B && q.numel() == (int64_t)B * H * D && out.size(0) == B &&
                   out.size(1) == H * Dv && window >= 1 && max_keys >= 1 && (!bias.has_value() || bias->numel() == H * window),
               "window_attn_decode: shapes disagree");
-  const int S = r32_window_attn_decode_splits(B, (int)G, (int)(H / G), (int)max_keys);
+  const int S = r32_window_attn_decode_splits(B, (int)G, (int)(H / G), (int)max_keys, D);
   auto part = torch::empty({(int64_t)B * H * S * (Dv + 2)}, q.options());
   float* po = part.data_ptr<float>();
   done(r32_window_attn_decode(q.data_ptr<float>(), k_cache.data_ptr(), v_cache.data_ptr(), (long long)k_cache.stride(0),
@@ -490,7 +492,9 @@ void gate_mul(Tensor a, Tensor g, int64_t mode) {
   done(r32_gate_mul(a.data_ptr(), lda, g.data_ptr(), ldg, (int)a.size(0), (int)a.size(1), (int)mode, f, stream()), "gate_mul");
 }
 
-void gated_norm_residual(Tensor x, Tensor y, c10::optional<Tensor> r, Tensor w, c10::optional<Tensor> x_cast, double eps) {
+// w_next (fp32 [d]): x_cast receives the NEXT sublayer's input norm of the new x, x / rms(x) * w_next, instead of a copy
+void gated_norm_residual(Tensor x, Tensor y, c10::optional<Tensor> r, Tensor w, c10::optional<Tensor> x_cast, double eps,
+                         c10::optional<Tensor> w_next) {
   want(x, torch::kFloat32, "gated_norm_residual x");
   want(w, torch::kFloat32, "gated_norm_residual w");
   const int fy = act_f32(y, "gated_norm_residual y");
@@ -511,8 +515,14 @@ void gated_norm_residual(Tensor x, Tensor y, c10::optional<Tensor> r, Tensor w, 
     TORCH_CHECK(x_cast->numel() == x.numel(), "gated_norm_residual: x_cast [T, d]");
     xc = x_cast->data_ptr();
   }
-  done(r32_gated_norm_residual(x.data_ptr<float>(), y.data_ptr(), ldy, rp, ldr, w.data_ptr<float>(), xc, T, d, (float)eps, fy,
-                               fr, stream()), "gated_norm_residual");
+  const float* wn = nullptr;
+  if (w_next.has_value()) {
+    want(*w_next, torch::kFloat32, "gated_norm_residual w_next");
+    TORCH_CHECK(w_next->numel() == d && xc != nullptr, "gated_norm_residual: w_next [d] needs x_cast");
+    wn = w_next->data_ptr<float>();
+  }
+  done(r32_gated_norm_residual(x.data_ptr<float>(), y.data_ptr(), ldy, rp, ldr, w.data_ptr<float>(), xc, wn, T, d, (float)eps,
+                               fy, fr, stream()), "gated_norm_residual");
 }
 
 void rmsnorm_rows(Tensor x, c10::optional<Tensor> rows, Tensor w, Tensor out, double eps) {
@@ -658,10 +668,24 @@ void latent_kv_write(Tensor proj, int64_t Cq, int64_t C, int64_t R, Tensor wq, T
 
 // q [T, H (D + R)] up-projected query rows; qn fp32 [H, T, C] their unrotated parts moved into the latent's space;
 // out fp32 [T, H, Dk] = [qn scale | rot(q_rot) scale | 0]
-void latent_q_rows(Tensor q, int64_t D, int64_t R, Tensor qn, Tensor freq, double mult, double scale, Tensor positions,
-                   Tensor out, int64_t H) {
+// qn absent: the unrotated part is the rows' own (q[:, h, :D] * scale), out [T, H, Dk >= D + R]
+void latent_q_rows(Tensor q, int64_t D, int64_t R, c10::optional<Tensor> qn_, Tensor freq, double mult, double scale,
+                   Tensor positions, Tensor out, int64_t H) {
   const int f = act_f32(q, "latent_q_rows q");
   const int ldq = row_stride(q, "latent_q_rows q");
+  if (!qn_.has_value()) {
+    want(freq, torch::kFloat32, "latent_q_rows freq");
+    want(positions, torch::kInt32, "latent_q_rows positions");
+    want(out, torch::kFloat32, "latent_q_rows out");
+    const int T = (int)q.size(0);
+    TORCH_CHECK(out.dim() == 3 && out.size(0) == T && out.size(1) == H && q.size(1) == H * (D + R) && R % 2 == 0 &&
+                    freq.numel() == R / 2 && positions.numel() == T && out.size(2) >= D + R, "latent_q_rows: shapes disagree");
+    done(r32_latent_q_rows(q.data_ptr(), ldq, (int)D, (int)R, nullptr, (int)D, freq.data_ptr<float>(), (float)mult, (float)scale,
+                           positions.data_ptr<int>(), out.data_ptr<float>(), (int)H, (int)out.size(2), T, f, stream()),
+         "latent_q_rows");
+    return;
+  }
+  Tensor qn = *qn_;
   want(qn, torch::kFloat32, "latent_q_rows qn");
   want(freq, torch::kFloat32, "latent_q_rows freq");
   want(positions, torch::kInt32, "latent_q_rows positions");
@@ -673,6 +697,27 @@ void latent_q_rows(Tensor q, int64_t D, int64_t R, Tensor qn, Tensor freq, doubl
   done(r32_latent_q_rows(q.data_ptr(), ldq, (int)D, (int)R, qn.data_ptr<float>(), (int)qn.size(2), freq.data_ptr<float>(),
                          (float)mult, (float)scale, positions.data_ptr<int>(), out.data_ptr<float>(), (int)H, (int)out.size(2), T,
                          f, stream()), "latent_q_rows");
+}
+
+// Keys and values up-projected from cached latents into pages of their own: kv rows [N, H D + H Dv] (keys of all heads,
+// then values), lat rows [N, >= rot_off + R] (the cached rows: the rotated key part at rot_off), slots int64 [N]; per
+// token and head the key row [kv key (D) | rotated part (R) | zeros] of dk entries, the value row [value | zeros] of dv.
+void latent_expand_write(Tensor kv, Tensor lat, int64_t rot_off, int64_t R, Tensor slots, Tensor k_cache, Tensor v_cache,
+                         int64_t H, int64_t D, int64_t Dv) {
+  const int f = act_f32(kv, "latent_expand_write kv");
+  const int ldk = row_stride(kv, "latent_expand_write kv"), ldl = row_stride(lat, "latent_expand_write lat");
+  want(slots, torch::kInt64, "latent_expand_write slots");
+  int NB, BS, nk, nv;
+  cache_layout(k_cache, v_cache, NB, BS, nk, nv, "latent_expand_write");
+  const int N = (int)kv.size(0);
+  TORCH_CHECK(lat.is_cuda() && lat.scalar_type() == kv.scalar_type() && k_cache.scalar_type() == kv.scalar_type() &&
+                  v_cache.scalar_type() == kv.scalar_type(), "latent_expand_write: one dtype");
+  TORCH_CHECK(H > 0 && nk % H == 0 && nv % H == 0 && kv.size(1) == H * (D + Dv) && lat.size(0) == N && lat.size(1) >= rot_off + R &&
+                  slots.numel() == N && nk / H >= D + R && nv / H >= Dv, "latent_expand_write: shapes disagree");
+  done(r32_latent_expand_write(kv.data_ptr(), ldk, lat.data_ptr(), ldl, (int)rot_off, (const long long*)slots.data_ptr<int64_t>(),
+                               k_cache.data_ptr(), v_cache.data_ptr(), (long long)k_cache.stride(0), (long long)v_cache.stride(0),
+                               BS, N, (int)H, (int)D, (int)R, (int)Dv, (int)(nk / H), (int)(nv / H), f, stream()),
+       "latent_expand_write");
 }
 
 int64_t retention_max_dim() { return r32_retention_max_dim(); }
@@ -750,6 +795,7 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
   m.def("moe_combine", &moe_combine);
   m.def("latent_kv_write", &latent_kv_write);
   m.def("latent_q_rows", &latent_q_rows);
+  m.def("latent_expand_write", &latent_expand_write);
   m.def("retention", &retention);
   m.def("retention_max_dim", &retention_max_dim);
   m.def("glu", &glu);

@@ -134,7 +134,7 @@ __global__ void gate_mul_vec_kernel(AT* __restrict__ a, int lda, const AT* __res
 template <typename YT, typename GT>
 __global__ void gated_norm_residual_kernel(float* __restrict__ x, const YT* __restrict__ y, int ldy,
                                            const GT* __restrict__ r, int ldr, const float* __restrict__ w,
-                                           bf16_t* __restrict__ x_cast, int d, float eps) {
+                                           bf16_t* __restrict__ x_cast, const float* __restrict__ w_next, int d, float eps) {
   __shared__ float scratch[16];
   const int t = blockIdx.x;
   const YT* yr = y + (size_t)t * ldy;
@@ -147,12 +147,18 @@ __global__ void gated_norm_residual_kernel(float* __restrict__ x, const YT* __re
   }
   const float rstd = 1.0f / sqrtf(block_sum(s, scratch) / (float)d + eps);
   float* xr = x + (size_t)t * d;
+  float s2 = 0.f;
   for (int i = threadIdx.x; i < d; i += blockDim.x) {
     float z = Elem<YT>::ld(yr + i);
     if (rr) z *= sigmoid_f(Elem<GT>::ld(rr + i));
     const float v = xr[i] + z * rstd * w[i];
     xr[i] = v;
-    if (x_cast) x_cast[(size_t)t * d + i] = f2bf(v);
+    s2 += v * v;
+    if (x_cast && !w_next) x_cast[(size_t)t * d + i] = f2bf(v);
+  }
+  if (x_cast && w_next) {  // the next sublayer's input norm of the new x (each thread re-reads what it wrote)
+    const float rstd2 = 1.0f / sqrtf(block_sum(s2, scratch) / (float)d + eps);
+    for (int i = threadIdx.x; i < d; i += blockDim.x) x_cast[(size_t)t * d + i] = f2bf(xr[i] * rstd2 * w_next[i]);
   }
 }
 
@@ -162,7 +168,8 @@ template <typename YT, typename GT, int NCH>
 __global__ void __launch_bounds__(256) gated_norm_residual_vec_kernel(float* __restrict__ x, const YT* __restrict__ y, int ldy,
                                                                        const GT* __restrict__ r, int ldr,
                                                                        const float* __restrict__ w,
-                                                                       bf16_t* __restrict__ x_cast, int d, float eps) {
+                                                                       bf16_t* __restrict__ x_cast,
+                                                                       const float* __restrict__ w_next, int d, float eps) {
   __shared__ float scratch[16];
   const int t = blockIdx.x;
   const YT* yr = y + (size_t)t * ldy;
@@ -184,13 +191,24 @@ __global__ void __launch_bounds__(256) gated_norm_residual_vec_kernel(float* __r
   }
   const float rstd = 1.0f / sqrtf(block_sum(s, scratch) / (float)d + eps);
   float* xr = x + (size_t)t * d;
+  float s2 = 0.f;
 #pragma unroll
   for (int u = 0; u < NCH; ++u) {
     const int i = (threadIdx.x + 256 * u) * 4;
     if (i < d) {
       const float4v v = Vec4<float>::ld(xr + i) + z[u] * rstd * Vec4<float>::ld(w + i);
       Vec4<float>::st(xr + i, v);
-      if (x_cast) Vec4<bf16_t>::st(x_cast + (size_t)t * d + i, v);
+      if (x_cast && !w_next) Vec4<bf16_t>::st(x_cast + (size_t)t * d + i, v);
+      z[u] = v;
+      s2 += v[0] * v[0] + v[1] * v[1] + v[2] * v[2] + v[3] * v[3];
+    }
+  }
+  if (x_cast && w_next) {  // the next sublayer's input norm of the new x, from registers
+    const float rstd2 = 1.0f / sqrtf(block_sum(s2, scratch) / (float)d + eps);
+#pragma unroll
+    for (int u = 0; u < NCH; ++u) {
+      const int i = (threadIdx.x + 256 * u) * 4;
+      if (i < d) Vec4<bf16_t>::st(x_cast + (size_t)t * d + i, z[u] * rstd2 * Vec4<float>::ld(w_next + i));
     }
   }
 }
@@ -205,6 +223,33 @@ __global__ void rmsnorm_rows_kernel(const float* __restrict__ x, const long long
   for (int i = threadIdx.x; i < d; i += blockDim.x) s += xr[i] * xr[i];
   const float rstd = 1.0f / sqrtf(block_sum(s, scratch) / (float)d + eps);
   for (int i = threadIdx.x; i < d; i += blockDim.x) Elem<AT>::st(out + (size_t)blockIdx.x * d + i, xr[i] * rstd * w[i]);
+}
+
+// d <= 4 * 256 * NCH, a multiple of four, aligned bases: the row is read once and stays in registers
+template <typename AT, int NCH>
+__global__ void __launch_bounds__(256) rmsnorm_rows_vec_kernel(const float* __restrict__ x, const long long* __restrict__ rows,
+                                                                const float* __restrict__ w, AT* __restrict__ out, int d,
+                                                                float eps) {
+  __shared__ float scratch[16];
+  const size_t r = rows ? (size_t)rows[blockIdx.x] : (size_t)blockIdx.x;
+  const float* xr = x + r * d;
+  float4v v[NCH];
+  float s = 0.f;
+#pragma unroll
+  for (int u = 0; u < NCH; ++u) {
+    const int i = (threadIdx.x + 256 * u) * 4;
+    v[u] = float4v{0.f, 0.f, 0.f, 0.f};
+    if (i < d) {
+      v[u] = Vec4<float>::ld(xr + i);
+      s += v[u][0] * v[u][0] + v[u][1] * v[u][1] + v[u][2] * v[u][2] + v[u][3] * v[u][3];
+    }
+  }
+  const float rstd = 1.0f / sqrtf(block_sum(s, scratch) / (float)d + eps);
+#pragma unroll
+  for (int u = 0; u < NCH; ++u) {
+    const int i = (threadIdx.x + 256 * u) * 4;
+    if (i < d) Vec4<AT>::st(out + (size_t)blockIdx.x * d + i, v[u] * rstd * Vec4<float>::ld(w + i));
+  }
 }
 
 template <typename AT>
@@ -314,21 +359,23 @@ extern "C" int r32_gate_mul(void* a, int lda, const void* g, int ldg, int T, int
 
 // y_f32 / r_f32: element types of the sublayer result and of the gate logits (r may be null: no gate)
 extern "C" int r32_gated_norm_residual(float* x, const void* y, int ldy, const void* r, int ldr, const float* w,
-                                       void* x_cast, int T, int d, float eps, int y_f32, int r_f32, hipStream_t s) {
+                                       void* x_cast, const float* w_next, int T, int d, float eps, int y_f32, int r_f32,
+                                       hipStream_t s) {
   if (T <= 0) return 0;
   const bool vec = d % 4 == 0 && d <= 8192 && ldy % 4 == 0 && ldr % 4 == 0 && aligned_to(x, 16) && aligned_to(w, 16) &&
+                   aligned_to(w_next, 16) &&
                    aligned_to(y, y_f32 ? 16 : 8) && aligned_to(r, r_f32 ? 16 : 8) && aligned_to(x_cast, 8);
   if (vec) {
     const int nch = (d + 1023) / 1024;
 #define LWC_GNR(YT, GT)                                                                                                  \
   if (nch <= 1)                                                                                                          \
-    gated_norm_residual_vec_kernel<YT, GT, 1><<<T, 256, 0, s>>>(x, (const YT*)y, ldy, (const GT*)r, ldr, w, (bf16_t*)x_cast, d, eps); \
+    gated_norm_residual_vec_kernel<YT, GT, 1><<<T, 256, 0, s>>>(x, (const YT*)y, ldy, (const GT*)r, ldr, w, (bf16_t*)x_cast, w_next, d, eps); \
   else if (nch <= 2)                                                                                                     \
-    gated_norm_residual_vec_kernel<YT, GT, 2><<<T, 256, 0, s>>>(x, (const YT*)y, ldy, (const GT*)r, ldr, w, (bf16_t*)x_cast, d, eps); \
+    gated_norm_residual_vec_kernel<YT, GT, 2><<<T, 256, 0, s>>>(x, (const YT*)y, ldy, (const GT*)r, ldr, w, (bf16_t*)x_cast, w_next, d, eps); \
   else if (nch <= 4)                                                                                                     \
-    gated_norm_residual_vec_kernel<YT, GT, 4><<<T, 256, 0, s>>>(x, (const YT*)y, ldy, (const GT*)r, ldr, w, (bf16_t*)x_cast, d, eps); \
+    gated_norm_residual_vec_kernel<YT, GT, 4><<<T, 256, 0, s>>>(x, (const YT*)y, ldy, (const GT*)r, ldr, w, (bf16_t*)x_cast, w_next, d, eps); \
   else                                                                                                                   \
-    gated_norm_residual_vec_kernel<YT, GT, 8><<<T, 256, 0, s>>>(x, (const YT*)y, ldy, (const GT*)r, ldr, w, (bf16_t*)x_cast, d, eps)
+    gated_norm_residual_vec_kernel<YT, GT, 8><<<T, 256, 0, s>>>(x, (const YT*)y, ldy, (const GT*)r, ldr, w, (bf16_t*)x_cast, w_next, d, eps)
     if (y_f32 && (r_f32 || !r)) {
       LWC_GNR(float, float);
     } else if (y_f32) {
@@ -343,11 +390,11 @@ extern "C" int r32_gated_norm_residual(float* x, const void* y, int ldy, const v
     return 0;
   }
   if (y_f32 && (r_f32 || !r))
-    gated_norm_residual_kernel<float, float><<<T, 256, 0, s>>>(x, (const float*)y, ldy, (const float*)r, ldr, w, (bf16_t*)x_cast, d, eps);
+    gated_norm_residual_kernel<float, float><<<T, 256, 0, s>>>(x, (const float*)y, ldy, (const float*)r, ldr, w, (bf16_t*)x_cast, w_next, d, eps);
   else if (y_f32)
-    gated_norm_residual_kernel<float, bf16_t><<<T, 256, 0, s>>>(x, (const float*)y, ldy, (const bf16_t*)r, ldr, w, (bf16_t*)x_cast, d, eps);
+    gated_norm_residual_kernel<float, bf16_t><<<T, 256, 0, s>>>(x, (const float*)y, ldy, (const bf16_t*)r, ldr, w, (bf16_t*)x_cast, w_next, d, eps);
   else if (!r_f32 || !r)
-    gated_norm_residual_kernel<bf16_t, bf16_t><<<T, 256, 0, s>>>(x, (const bf16_t*)y, ldy, (const bf16_t*)r, ldr, w, (bf16_t*)x_cast, d, eps);
+    gated_norm_residual_kernel<bf16_t, bf16_t><<<T, 256, 0, s>>>(x, (const bf16_t*)y, ldy, (const bf16_t*)r, ldr, w, (bf16_t*)x_cast, w_next, d, eps);
   else
     return -1;
   LWC_CHECK_LAUNCH();
@@ -357,6 +404,22 @@ extern "C" int r32_gated_norm_residual(float* x, const void* y, int ldy, const v
 extern "C" int r32_rmsnorm_rows(const float* x, const long long* rows, const float* w, void* out, int n, int d, float eps,
                                 int f32, hipStream_t s) {
   if (n <= 0) return 0;
+  if (d % 4 == 0 && d <= 8192 && aligned_to(x, 16) && aligned_to(w, 16) && aligned_to(out, f32 ? 16 : 8)) {
+    const int nch = (d + 1023) / 1024;
+#define LWC_RMS(AT)                                                                                  \
+  if (nch <= 1) rmsnorm_rows_vec_kernel<AT, 1><<<n, 256, 0, s>>>(x, rows, w, (AT*)out, d, eps);      \
+  else if (nch <= 2) rmsnorm_rows_vec_kernel<AT, 2><<<n, 256, 0, s>>>(x, rows, w, (AT*)out, d, eps); \
+  else if (nch <= 4) rmsnorm_rows_vec_kernel<AT, 4><<<n, 256, 0, s>>>(x, rows, w, (AT*)out, d, eps); \
+  else rmsnorm_rows_vec_kernel<AT, 8><<<n, 256, 0, s>>>(x, rows, w, (AT*)out, d, eps)
+    if (f32) {
+      LWC_RMS(float);
+    } else {
+      LWC_RMS(bf16_t);
+    }
+#undef LWC_RMS
+    LWC_CHECK_LAUNCH();
+    return 0;
+  }
   if (f32) rmsnorm_rows_kernel<float><<<n, 256, 0, s>>>(x, rows, w, (float*)out, d, eps);
   else rmsnorm_rows_kernel<bf16_t><<<n, 256, 0, s>>>(x, rows, w, (bf16_t*)out, d, eps);
   LWC_CHECK_LAUNCH();

@@ -77,7 +77,8 @@ latent_q_rows_kernel(const AT* __restrict__ q, int ldq, int D, int R, const floa
   float* o = out + (size_t)t * H * Dk;
   for (int e = threadIdx.x; e < H * C; e += blockDim.x) {
     const int h = e / C, i = e - h * C;
-    o[(size_t)h * Dk + i] = qn[((size_t)h * T + t) * C + i] * scale;
+    // without qn the unrotated part is the row's own (C == D then)
+    o[(size_t)h * Dk + i] = (qn ? qn[((size_t)h * T + t) * C + i] : Elem<AT>::ld(q + (size_t)t * ldq + (size_t)h * (D + R) + i)) * scale;
   }
   for (int e = threadIdx.x; e < H * (R / 2); e += blockDim.x) {
     const int h = e / (R / 2), i = e - h * (R / 2);
@@ -96,10 +97,55 @@ latent_q_rows_kernel(const AT* __restrict__ q, int ldq, int D, int R, const floa
   }
 }
 
+// One workgroup per token: key rows [H][dk] = [kv key of the head (D) | the token's rotated part (R) | 0], value rows
+// [H][dv] = [kv value | 0] in the 4-token interleaved layout.
+template <typename AT>
+__global__ void __launch_bounds__(256)
+latent_expand_write_kernel(const AT* __restrict__ kv, int ldk, const AT* __restrict__ lat, int ldl, int rot_off,
+                           const long long* __restrict__ slots, AT* __restrict__ k_cache, AT* __restrict__ v_cache,
+                           long long kb_stride, long long vb_stride, int block_size, int H, int D, int R, int Dv, int dk, int dv) {
+  const int t = blockIdx.x;
+  const long long slot = slots[t];
+  if (slot < 0) return;
+  const long long blk = slot / block_size, off = slot % block_size;
+  const AT* kr = kv + (size_t)t * ldk;
+  const AT* lr = lat + (size_t)t * ldl + rot_off;
+  AT* kc = k_cache + blk * kb_stride + off * ((long long)H * dk);
+  AT* vc = v_cache + blk * vb_stride + (off >> 2) * (4LL * H * dv) + (off & 3);
+  for (int e = threadIdx.x; e < H * dk; e += blockDim.x) {
+    const int h = e / dk, i = e - h * dk;
+    AT v = 0;
+    if (i < D) v = kr[h * D + i];
+    else if (i < D + R) v = lr[i - D];
+    kc[e] = v;
+  }
+  for (int e = threadIdx.x; e < H * dv; e += blockDim.x) {
+    const int h = e / dv, i = e - h * dv;
+    vc[4 * e] = i < Dv ? kr[H * D + h * Dv + i] : (AT)0;
+  }
+}
+
 }  // namespace
 }  // namespace lwc
 
 using namespace lwc;
+
+extern "C" int r32_latent_expand_write(const void* kv, int ldk, const void* lat, int ldl, int rot_off, const long long* slots,
+                                       void* k_cache, void* v_cache, long long kb_stride, long long vb_stride, int block_size,
+                                       int N, int H, int D, int R, int Dv, int dk, int dv, int f32, hipStream_t s) {
+  if (N <= 0) return 0;
+  if (dk < D + R || dv < Dv) return -1;
+  if (f32)
+    latent_expand_write_kernel<float><<<N, 256, 0, s>>>((const float*)kv, ldk, (const float*)lat, ldl, rot_off, slots,
+                                                        (float*)k_cache, (float*)v_cache, kb_stride, vb_stride, block_size, H, D,
+                                                        R, Dv, dk, dv);
+  else
+    latent_expand_write_kernel<bf16_t><<<N, 256, 0, s>>>((const bf16_t*)kv, ldk, (const bf16_t*)lat, ldl, rot_off, slots,
+                                                         (bf16_t*)k_cache, (bf16_t*)v_cache, kb_stride, vb_stride, block_size,
+                                                         H, D, R, Dv, dk, dv);
+  LWC_CHECK_LAUNCH();
+  return 0;
+}
 
 extern "C" int r32_latent_kv_write(const void* proj, int ldp, int Cq, int C, int R, const float* wq, const float* wc,
                                    const float* freq, float mult, const int* positions, const int* slots, void* cq, int ldq,

@@ -40,14 +40,18 @@ struct WAttnDecodeParams {
   int H, G, S, keys_per_split;  // keys_per_split: a multiple of 32
 };
 
-template <int ND, int NV>
-__global__ void __launch_bounds__(64) window_attn_decode_kernel(const WAttnDecodeParams p) {
-  constexpr int D = 32 * ND, DV = 16 * NV;
+// NW waves per workgroup share one (sequence, head chunk, split): every wave forms the scores of all keys itself and
+// owns NV / NW of the 16-column value tiles (wide value rows: the accumulators of one wave would leave no registers
+// for loads in flight).  QLO = false: q enters as its bf16 rounding only (one MFMA per operand instead of two).
+template <int ND, int NV, int NW = 1, bool QLO = true>
+__global__ void __launch_bounds__(64 * NW) window_attn_decode_kernel(const WAttnDecodeParams p) {
+  constexpr int D = 32 * ND, DV = 16 * NV, NVW = NV / NW;
+  static_assert(NV % NW == 0, "value tiles divide among the waves");
   const int b = blockIdx.x, split = blockIdx.z;
   const int H = p.H, G = p.G, Hg = H / G, chunks = (Hg + 15) / 16;
   const int g = blockIdx.y / chunks, h0 = g * Hg + (blockIdx.y % chunks) * 16;
   const int nh = min(16, g * Hg + Hg - h0);  // heads of this chunk
-  const int lane = threadIdx.x, r16 = lane & 15, g4 = lane >> 4;
+  const int lane = threadIdx.x & 63, wv = threadIdx.x >> 6, r16 = lane & 15, g4 = lane >> 4;
   const int i = p.positions[b];
   const int j_lo = max(0, i - p.window + 1);
   const int base = (j_lo / 32) * 32 + split * p.keys_per_split;  // this split's first key (a multiple of 32)
@@ -66,7 +70,7 @@ __global__ void __launch_bounds__(64) window_attn_decode_kernel(const WAttnDecod
   const bool h_valid = r16 < nh;
   const int h = h0 + (h_valid ? r16 : 0);
 
-  short8 qhi[ND], qlo[ND];
+  short8 qhi[ND], qlo[QLO ? ND : 1];
 #pragma unroll
   for (int kd = 0; kd < ND; ++kd) {
 #pragma unroll
@@ -75,12 +79,12 @@ __global__ void __launch_bounds__(64) window_attn_decode_kernel(const WAttnDecod
       if (h_valid) x = p.q[((size_t)b * H + h) * D + kd * 32 + 8 * g4 + e];
       const bf16_t hi = f2bf(x);
       qhi[kd][e] = (short)hi;
-      qlo[kd][e] = (short)f2bf(x - bf2f(hi));
+      if (QLO) qlo[kd][e] = (short)f2bf(x - bf2f(hi));
     }
   }
-  float4v O[NV];
+  float4v O[NVW];
 #pragma unroll
-  for (int n = 0; n < NV; ++n) O[n] = float4v{0.f, 0.f, 0.f, 0.f};
+  for (int n = 0; n < NVW; ++n) O[n] = float4v{0.f, 0.f, 0.f, 0.f};
   float m = -1e30f, l = 0.f;
   const float* bias_h = p.bias ? p.bias + (size_t)h * p.window : nullptr;  // no table: no distance bias
 
@@ -95,7 +99,7 @@ __global__ void __launch_bounds__(64) window_attn_decode_kernel(const WAttnDecod
       for (int kd = 0; kd < ND; ++kd) {
         const short8 a = *reinterpret_cast<const short8*>(kr + kd * 32);
         sacc[sub] = mfma16(a, qhi[kd], sacc[sub]);
-        sacc[sub] = mfma16(a, qlo[kd], sacc[sub]);
+        if (QLO) sacc[sub] = mfma16(a, qlo[kd], sacc[sub]);
       }
     }
     float s[8];
@@ -139,11 +143,11 @@ __global__ void __launch_bounds__(64) window_attn_decode_kernel(const WAttnDecod
     const bf16_t* va = p.v_cache + (long long)page_of(ja) * p.vb_stride + (long long)(page_off(ja) >> 2) * (4LL * G * DV) + 4LL * (g * DV + r16);
     const bf16_t* vb = p.v_cache + (long long)page_of(jb) * p.vb_stride + (long long)(page_off(jb) >> 2) * (4LL * G * DV) + 4LL * (g * DV + r16);
 #pragma unroll
-    for (int n = 0; n < NV; ++n) {
+    for (int n = 0; n < NVW; ++n) {
 #pragma unroll
       for (int r = 0; r < 4; ++r) O[n][r] *= ar[r];
-      const short4v b0 = *reinterpret_cast<const short4v*>(va + 64 * n);
-      const short4v b1 = *reinterpret_cast<const short4v*>(vb + 64 * n);
+      const short4v b0 = *reinterpret_cast<const short4v*>(va + 64 * (wv * NVW + n));
+      const short4v b1 = *reinterpret_cast<const short4v*>(vb + 64 * (wv * NVW + n));
       const short8 bb = short8{b0[0], b0[1], b0[2], b0[3], b1[0], b1[1], b1[2], b1[3]};
       O[n] = mfma16(ph, bb, O[n]);
       O[n] = mfma16(pl, bb, O[n]);
@@ -156,10 +160,10 @@ __global__ void __launch_bounds__(64) window_attn_decode_kernel(const WAttnDecod
     if (hr < nh) {
       float* po = p.part_o + (((size_t)b * H + h0 + hr) * p.S + split) * DV;
 #pragma unroll
-      for (int n = 0; n < NV; ++n) po[n * 16 + r16] = O[n][r];
+      for (int n = 0; n < NVW; ++n) po[(wv * NVW + n) * 16 + r16] = O[n][r];
     }
   }
-  if (g4 == 0 && h_valid) {
+  if (g4 == 0 && h_valid && wv == 0) {
     float* pm = p.part_ml + (((size_t)b * H + h) * p.S + split) * 2;
     pm[0] = m;
     pm[1] = l;
@@ -203,10 +207,12 @@ int launch_decode_nv(const WAttnDecodeParams& p, int nv, dim3 grid, hipStream_t 
 // Splits for a decode step of B sequences whose windows hold at most max_keys keys: about 2048 waves (two per SIMD),
 // at least 64 keys each.  Measured at 64 sequences x 8 kv heads x 2048 keys of 128: 3 splits 150 us, 4 splits
 // (2048 waves) 130 us, 8 splits 155 us, 16 splits 146 us (shorter key runs per wave, larger partials to merge).
-extern "C" int r32_window_attn_decode_splits(int B, int G, int Hg, int max_keys) {
+// Wide rows (D = 576): workgroups of four waves, about 1024 of them, at least 128 keys each (their partials are large).
+extern "C" int r32_window_attn_decode_splits(int B, int G, int Hg, int max_keys, int D) {
   const int waves = B * G * ((Hg + 15) / 16);
-  int s = (2048 + waves - 1) / waves;
-  const int by_keys = (max_keys + 32 + 63) / 64;
+  const bool wide = D > 128;
+  int s = ((wide ? 1024 : 2048) + waves - 1) / waves;
+  const int by_keys = wide ? (max_keys + 32 + 127) / 128 : (max_keys + 32 + 63) / 64;
   if (s > by_keys) s = by_keys;
   if (s > 64) s = 64;
   return s < 1 ? 1 : s;
@@ -235,7 +241,7 @@ extern "C" int r32_window_attn_decode(const float* q, const void* k_cache, const
   const dim3 grid(B, G * ((Hg + 15) / 16), S);
   int rc = -1;
   if (D == 576 && Dv == 512) {  // one wide row for all heads: a low-rank attention's cached latent + rotated part
-    window_attn_decode_kernel<18, 32><<<grid, 64, 0, s>>>(p);
+    window_attn_decode_kernel<18, 32, 4, false><<<grid, 256, 0, s>>>(p);
     rc = (int)hipGetLastError();
   } else {
     switch (D / 32) {

@@ -398,20 +398,12 @@ class LimatarModel:
         rows = k_rows[ctx["blk"], ctx["off"]]                                      # [N, row]: latent | rotated part
         N = rows.shape[0]
         kv = F.linear(rows[:, :C], x["w_ukv"])                                     # [N, H D + H Dv]
-        kexp = torch.zeros(N, H, dk, dtype=self.dtype, device=self.device)
-        kexp[:, :, :D] = kv[:, :H * D].view(N, H, D)
-        kexp[:, :, D:D + R] = rows[:, None, C:C + R]
-        vexp = kv[:, H * D:]
-        if dv != Dv:
-            vexp = torch.zeros(N, H, dv, dtype=self.dtype, device=self.device)
-            vexp[:, :, :Dv] = kv[:, H * D:].view(N, H, Dv)
         key = ("pages", H * dk, H * dv)
         tmp = plan.scratch.get(key)
         if tmp is None:
             tmp = plan.scratch[key] = PagedLayerCache([(H * dk, H * dv)], ctx["pages"], bs, self.device, self.dtype)
-        tmp.set_rows(0, ctx["slots"], kexp.view(N, H * dk), vexp.reshape(N, H * dv))
-        qn = q.view(Tq, H, D + R)[:, :, :D].permute(1, 0, 2).float().contiguous()   # [H, Tq, D]
-        qf = res32.latent_q_rows(q, D, R, qn, x["freq"], x["rot_mult"], m.scale, positions, H, dk)
+        res32.latent_expand_write(kv, rows, C, R, ctx["slots"], tmp.k[0], tmp.v[0], H, D, Dv)
+        qf = res32.latent_q_rows(q, D, R, None, x["freq"], x["rot_mult"], m.scale, positions, H, dk)
         out = torch.empty(Tq, H * dv, dtype=self.dtype, device=self.device)
         ch, z = plan.chunk, self._no_bias(H)
         res32.window_attn(qf.view(Tq, H * dk), tmp.k[0], tmp.v[0], positions, ctx["tables"], z, z, UNBOUNDED, out, H, H,
@@ -460,22 +452,41 @@ class LimatarModel:
         output projection and the feed-forward on the kept rows only; returns [len(keep), d]."""
         cfg, dt, eps = self.cfg, self.dtype, self.cfg.norm_eps
         x = res32.rmsnorm_rows(res32.embed_rows(self.embed, tokens), self.embed_norm, eps, torch.float32)
+        n = len(self.runs)
+        h = res32.rmsnorm_rows(x, self.layers[self.runs[0]].norm1, eps, dt) if n else None
         for ri, li in enumerate(self.runs):
             S, L = cfg.layer_specs[li], self.layers[li]
-            h = res32.rmsnorm_rows(x, L.norm1, eps, dt)
             if S.type == "latent_attention":
                 a = self._latent_mixer(h, L, S.mixer, ri, positions, slots, cache, plan)
             else:
                 a = self._retention_mixer(h, L, S.mixer, ri, state, items)
-            if keep is not None and ri + 1 == len(self.runs):   # from here on only the kept rows
+            last = ri + 1 == n
+            if keep is not None and last:   # from here on only the kept rows
                 a, x = a.index_select(0, keep), x.index_select(0, keep)
-            res32.gated_norm_residual(x, self._linear(a, L.w_o), L.norm1b, eps)
+            nxt = None if last else self.layers[self.runs[ri + 1]].norm1
+            y = self._linear(a, L.w_o)
             if S.mlp is not None:
-                h2 = res32.rmsnorm_rows(x, L.norm2, eps, dt)
-                res32.gated_norm_residual(x, self._feed_forward(h2, L, S.mlp), L.norm2b, eps)
+                h2 = self._add_norm(x, y, L.norm1b, L.norm2)
+                h = self._add_norm(x, self._feed_forward(h2, L, S.mlp), L.norm2b, nxt)
+            else:
+                h = self._add_norm(x, y, L.norm1b, nxt)
             if self.on_layer is not None:
                 self.on_layer(ri, x)
         return x
+
+    def _add_norm(self, x: torch.Tensor, y: torch.Tensor, w: torch.Tensor, next_w: Optional[torch.Tensor]):
+        """x += y / rms(y) * w; returns the next sublayer's input x / rms(x) * next_w (None without ``next_w``): one
+        pass over the stream in bf16 (the new x stays in registers between the two norms)."""
+        eps = self.cfg.norm_eps
+        if next_w is None:
+            res32.gated_norm_residual(x, y, w, eps)
+            return None
+        if self.dtype == torch.bfloat16:
+            h = torch.empty(x.shape[0], x.shape[1], dtype=self.dtype, device=self.device)
+            res32.gated_norm_residual(x, y, w, eps, x_cast=h, next_w=next_w)
+            return h
+        res32.gated_norm_residual(x, y, w, eps)
+        return res32.rmsnorm_rows(x, next_w, eps, self.dtype)
 
     def _logits(self, x: torch.Tensor, rows: Optional[torch.Tensor], float_logits: bool) -> torch.Tensor:
         h = res32.rmsnorm_rows(x, self.final_w, self.cfg.norm_eps, self.dtype, rows=rows)

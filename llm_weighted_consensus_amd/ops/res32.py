@@ -218,10 +218,12 @@ def gate_mul(a: torch.Tensor, g: torch.Tensor, mode: str = "sigmoid") -> torch.T
 
 
 def gated_norm_residual(x: torch.Tensor, y: torch.Tensor, w: torch.Tensor, eps: float,
-                        gate_logits: Optional[torch.Tensor] = None, x_cast: Optional[torch.Tensor] = None) -> None:
+                        gate_logits: Optional[torch.Tensor] = None, x_cast: Optional[torch.Tensor] = None,
+                        next_w: Optional[torch.Tensor] = None) -> None:
     """x (fp32) += z / rms(z) * w with z = y * sigmoid(gate_logits) (z = y without); w fp32.  ``x_cast`` (bf16
-    [T, d]) also receives the new x."""
-    kernels().gated_norm_residual(x, y, gate_logits, w, x_cast, float(eps))
+    [T, d]) also receives the new x, or with ``next_w`` (fp32 [d]) the next sublayer's input norm of it,
+    x / rms(x) * next_w."""
+    kernels().gated_norm_residual(x, y, gate_logits, w, x_cast, float(eps), next_w)
 
 
 def rmsnorm_rows(x: torch.Tensor, w: torch.Tensor, eps: float, dtype, rows: Optional[torch.Tensor] = None) -> torch.Tensor:
@@ -304,13 +306,22 @@ def latent_kv_write(proj: torch.Tensor, Cq: int, C: int, R: int, wq: torch.Tenso
     return cq
 
 
-def latent_q_rows(q: torch.Tensor, D: int, R: int, qn: torch.Tensor, freq: torch.Tensor, mult: float, scale: float,
+def latent_q_rows(q: torch.Tensor, D: int, R: int, qn: Optional[torch.Tensor], freq: torch.Tensor, mult: float, scale: float,
                   positions: torch.Tensor, H: int, Dk: int) -> torch.Tensor:
     """fp32 query rows [T, H, Dk] of a low-rank attention layer: per head [qn * scale | rot(q[:, D : D + R]) * mult *
-    scale | 0], ``qn`` fp32 [H, T, C] = the unrotated query parts times the keys' up-projection."""
+    scale | 0], ``qn`` fp32 [H, T, C] = the unrotated query parts times the keys' up-projection; ``qn`` None: the
+    unrotated parts themselves (q[:, :D] of every head)."""
     out = torch.empty(q.shape[0], H, Dk, dtype=torch.float32, device=q.device)
     kernels().latent_q_rows(q, int(D), int(R), qn, freq, float(mult), float(scale), positions, out, int(H))
     return out
+
+
+def latent_expand_write(kv: torch.Tensor, lat: torch.Tensor, rot_off: int, R: int, slots: torch.Tensor, k_cache: torch.Tensor,
+                        v_cache: torch.Tensor, H: int, D: int, Dv: int) -> None:
+    """Keys and values up-projected from cached latents, written as pages of their own: ``kv`` [N, H D + H Dv], ``lat``
+    the tokens' cached rows (their rotated key part at ``rot_off``), ``slots`` int64 [N].  Per token and head the key
+    row is [key (D) | rotated part (R) | zeros], the value row [value (Dv) | zeros] (4-token interleaved)."""
+    kernels().latent_expand_write(kv, lat, int(rot_off), int(R), slots, k_cache, v_cache, int(H), int(D), int(Dv))
 
 
 def retention(proj: torch.Tensor, k_off: int, v: torch.Tensor, freq: torch.Tensor, mult: float, rot_dims: int,

@@ -86,6 +86,36 @@ def test_latent_cache_rows_and_query_rows(gpu, dtype, tol, H, D, R, C, Cq):
     assert (qf[..., :C] - qn.double().transpose(0, 1) * scale).abs().max() < 1e-5
     assert (qf[..., C:C + R] - ref_rot).abs().max() < 2e-5 * max(1.0, float(ref_rot.abs().max()))
     assert float(qf[..., C + R:].abs().sum()) == 0
+    # without the absorbed part: the rows' own unrotated entries (attention over up-projected keys)
+    Dq = -(-(D + R) // 32) * 32
+    q2 = res32.latent_q_rows(q.to(gpu), D, R, None, f, m, scale, pos.to(gpu), H, Dq).cpu().double()
+    assert (q2[..., :D] - q.double().view(T, H, D + R)[..., :D] * scale).abs().max() < 1e-5
+    assert (q2[..., D:D + R] - ref_rot).abs().max() < 2e-5 * max(1.0, float(ref_rot.abs().max()))
+    assert float(q2[..., D + R:].abs().sum()) == 0
+
+
+@pytest.mark.parametrize("d", [44, 64, 1028, 4096])
+def test_residual_add_with_both_norms_in_one_pass(gpu, d):
+    """x += norm(y) (1 + w) and, in the same pass, the next sublayer's input norm of the new x (bf16 rows), against the
+    oracle; the plain row norm (fp32 and bf16 rows, gathered rows) beside it."""
+    from llm_weighted_consensus_amd.ops import res32
+
+    g = torch.Generator().manual_seed(d)
+    T, eps = 9, 1e-5
+    x, y = torch.randn(T, d, generator=g) * 3, torch.randn(T, d, generator=g).to(torch.bfloat16)
+    w, wn = 0.1 * torch.randn(d, generator=g), 0.1 * torch.randn(d, generator=g)
+    ref_x = x.double() + O.norm_zero_centered(y.double(), w, eps)
+    ref_h = O.norm_zero_centered(ref_x, wn, eps)
+    xg, h = x.to(gpu), torch.empty(T, d, dtype=torch.bfloat16, device=gpu)
+    res32.gated_norm_residual(xg, y.to(gpu), (1 + w).to(gpu), eps, x_cast=h, next_w=(1 + wn).to(gpu))
+    assert (xg.cpu().double() - ref_x).abs().max() < 1e-5 * 8
+    assert (h.cpu().double() - ref_h).abs().max() < 3e-2
+    rows = torch.tensor([4, 0, 8])
+    for dt, tol in ((torch.float32, 1e-5), (torch.bfloat16, 3e-2)):
+        got = res32.rmsnorm_rows(xg, (1 + wn).to(gpu), eps, dt).cpu().double()
+        assert (got - ref_h).abs().max() < tol * 4
+        got = res32.rmsnorm_rows(xg, (1 + wn).to(gpu), eps, dt, rows=rows.to(gpu)).cpu().double()
+        assert (got - ref_h[rows]).abs().max() < tol * 4
 
 
 def _paged(n_tokens, bs, nk, nv, dtype, gpu, seed=0):
@@ -369,7 +399,7 @@ def _err(got, ref, dtype=torch.float32):
     return 4 * float(rel.flatten().quantile(0.9))
 
 
-TOL = {torch.float32: 1e-4, torch.bfloat16: 0.5}
+TOL = {torch.float32: 3e-4, torch.bfloat16: 0.5}
 
 
 @pytest.mark.parametrize("name,dtype", [(n, d) for d in (torch.float32, torch.bfloat16) for n in ("mixed", "odd", "recurrent", "attentive", "wide", "deep")
