@@ -42,7 +42,9 @@ struct WAttnDecodeParams {
 
 // NW waves per workgroup share one (sequence, head chunk, split): every wave forms the scores of all keys itself and
 // owns NV / NW of the 16-column value tiles (wide value rows: the accumulators of one wave would leave no registers
-// for loads in flight).  QLO = false: q enters as its bf16 rounding only (one MFMA per operand instead of two).
+// for loads in flight).  With NW > 1 a tile's 32 key rows go through LDS once for all the waves (fetched into registers
+// one tile ahead); a wave's own value words still come straight from the cache.  QLO = false: q enters as its bf16
+// rounding only (one MFMA per operand instead of two).
 template <int ND, int NV, int NW = 1, bool QLO = true>
 __global__ void __launch_bounds__(64 * NW) window_attn_decode_kernel(const WAttnDecodeParams p) {
   constexpr int D = 32 * ND, DV = 16 * NV, NVW = NV / NW;
@@ -51,7 +53,9 @@ __global__ void __launch_bounds__(64 * NW) window_attn_decode_kernel(const WAttn
   const int H = p.H, G = p.G, Hg = H / G, chunks = (Hg + 15) / 16;
   const int g = blockIdx.y / chunks, h0 = g * Hg + (blockIdx.y % chunks) * 16;
   const int nh = min(16, g * Hg + Hg - h0);  // heads of this chunk
-  const int lane = threadIdx.x & 63, wv = threadIdx.x >> 6, r16 = lane & 15, g4 = lane >> 4;
+  // (one wave: the wave index is a compile-time zero, so the value tiles' offsets stay immediates)
+  const int lane = NW > 1 ? (int)(threadIdx.x & 63) : (int)threadIdx.x, wv = NW > 1 ? (int)(threadIdx.x >> 6) : 0;
+  const int r16 = lane & 15, g4 = lane >> 4;
   const int i = p.positions[b];
   const int j_lo = max(0, i - p.window + 1);
   const int base = (j_lo / 32) * 32 + split * p.keys_per_split;  // this split's first key (a multiple of 32)
@@ -88,18 +92,56 @@ __global__ void __launch_bounds__(64 * NW) window_attn_decode_kernel(const WAttn
   float m = -1e30f, l = 0.f;
   const float* bias_h = p.bias ? p.bias + (size_t)h * p.window : nullptr;  // no table: no distance bias
 
-  for (int t0 = base; t0 <= last; t0 += 32) {
+  constexpr bool kStage = NW > 1;
+  constexpr int KLD = D + 8;                                       // LDS row stride: rows start in different banks
+  constexpr int KCH = (32 * (D / 8) + 64 * NW - 1) / (64 * NW);    // 16-byte words per thread and tile
+  __shared__ __attribute__((aligned(16))) bf16_t K_s[kStage ? 32 * KLD : 8];
+  uint4v kreg[kStage ? KCH : 1];
+  auto fetch = [&](int t0) {
+#pragma unroll
+    for (int u = 0; u < KCH; ++u) {
+      const int c = (int)threadIdx.x + 64 * NW * u;
+      const int key = c / (D / 8), dc = c % (D / 8);
+      const int j = min(t0 + min(key, 31), i);  // (rows past the token are masked below: any valid row does)
+      kreg[u] = *reinterpret_cast<const uint4v*>(p.k_cache + (long long)page_of(j) * p.kb_stride +
+                                                 ((long long)page_off(j) * G + g) * D + dc * 8);
+    }
+  };
+  auto stash = [&]() {
+#pragma unroll
+    for (int u = 0; u < KCH; ++u) {
+      const int c = (int)threadIdx.x + 64 * NW * u;
+      if (c < 32 * (D / 8)) *reinterpret_cast<uint4v*>(&K_s[(c / (D / 8)) * KLD + (c % (D / 8)) * 8]) = kreg[u];
+    }
+  };
+  if (kStage && base <= last) {
+    fetch(base);
+    stash();
+    __syncthreads();
+  }
+
+  for (int t0 = base; t0 <= last; t0 += 32) {  // (base and last are the same for every wave of the workgroup)
+    if (kStage && t0 + 32 <= last) fetch(t0 + 32);
     float4v sacc[2];
 #pragma unroll
     for (int sub = 0; sub < 2; ++sub) {
       sacc[sub] = float4v{0.f, 0.f, 0.f, 0.f};
-      const int j = min(t0 + sub * 16 + r16, i);  // (rows past the token are masked below: any valid row does)
-      const bf16_t* kr = p.k_cache + (long long)page_of(j) * p.kb_stride + ((long long)page_off(j) * G + g) * D + 8 * g4;
+      if (kStage) {
 #pragma unroll
-      for (int kd = 0; kd < ND; ++kd) {
-        const short8 a = *reinterpret_cast<const short8*>(kr + kd * 32);
-        sacc[sub] = mfma16(a, qhi[kd], sacc[sub]);
-        if (QLO) sacc[sub] = mfma16(a, qlo[kd], sacc[sub]);
+        for (int kd = 0; kd < ND; ++kd) {
+          const short8 a = *reinterpret_cast<const short8*>(&K_s[(sub * 16 + r16) * KLD + kd * 32 + 8 * g4]);
+          sacc[sub] = mfma16(a, qhi[kd], sacc[sub]);
+          if (QLO) sacc[sub] = mfma16(a, qlo[kd], sacc[sub]);
+        }
+      } else {
+        const int j = min(t0 + sub * 16 + r16, i);  // (rows past the token are masked below: any valid row does)
+        const bf16_t* kr = p.k_cache + (long long)page_of(j) * p.kb_stride + ((long long)page_off(j) * G + g) * D + 8 * g4;
+#pragma unroll
+        for (int kd = 0; kd < ND; ++kd) {
+          const short8 a = *reinterpret_cast<const short8*>(kr + kd * 32);
+          sacc[sub] = mfma16(a, qhi[kd], sacc[sub]);
+          if (QLO) sacc[sub] = mfma16(a, qlo[kd], sacc[sub]);
+        }
       }
     }
     float s[8];
@@ -151,6 +193,11 @@ __global__ void __launch_bounds__(64 * NW) window_attn_decode_kernel(const WAttn
       const short8 bb = short8{b0[0], b0[1], b0[2], b0[3], b1[0], b1[1], b1[2], b1[3]};
       O[n] = mfma16(ph, bb, O[n]);
       O[n] = mfma16(pl, bb, O[n]);
+    }
+    if (kStage) {
+      __syncthreads();  // every wave has read this tile's rows
+      if (t0 + 32 <= last) stash();
+      __syncthreads();
     }
   }
   // partials: O rows are heads 4 g4 + r, columns dv 16 n + r16

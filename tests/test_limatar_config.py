@@ -88,10 +88,7 @@ def test_oracle_mechanisms_agree_with_their_definitions():
     for rotate in (O.rotate_interleaved, O.rotate_half):
         a, b = rotate(q, cos, sin), rotate(k, cos, sin)
         assert (a.norm(dim=-1) - q.norm(dim=-1)).abs().max() < 1e-12
-        c3, s3 = O.rope_tables(rot, torch.tensor([3]))
-        shifted = rotate(k[2:3], c3, s3)  # k of token 2 as if it stood 3 positions later
-        assert abs(float((a[6, 0] * b[2, 0]).sum()) - float((a[6 + 0, 0] * b[2, 0]).sum())) < 1e-12
-        c9, s9 = O.rope_tables(rot, torch.tensor([4]))
-        assert abs(float((rotate(q[6:7], c9, s9)[0, 0] * rotate(k[2:3], *O.rope_tables(rot, torch.tensor([0])))[0, 0]).sum())
-                   - float((a[6, 0] * b[2, 0]).sum())) < 1e-9  # only the distance 6 - 2 matters
-        del shifted
+        c4, s4 = O.rope_tables(rot, torch.tensor([4]))
+        c0, s0 = O.rope_tables(rot, torch.tensor([0]))
+        moved = float((rotate(q[6:7], c4, s4)[0, 0] * rotate(k[2:3], c0, s0)[0, 0]).sum())
+        assert abs(moved - float((a[6, 0] * b[2, 0]).sum())) < 1e-9  # only the distance 6 - 2 matters
