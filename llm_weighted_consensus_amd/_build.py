@@ -68,7 +68,7 @@ def _torch_flags(name: str = "_kernels") -> tuple[list[str], list[str]]:
 # compiler's default AGPR form moved every O accumulator AGPR <-> VGPR around each MFMA: 72 v_accvgpr per
 # 32-key tile).
 PER_FILE_FLAGS = {f: ["-mllvm", "-amdgpu-mfma-vgpr-form=1"] for f in ("attention_prefill.hip", "attention_decode.hip",
-                                                                      "wattn.hip")}
+                                                                      "wattn.hip", "wattn_decode_wide.hip")}
 
 
 def build_kernels(jobs: int = 8, force: bool = False) -> Path:

@@ -14,16 +14,18 @@ is formed once at load).  A layer run over the T rows of a step (decode rows and
                                                          against the cached latent itself
       o_c  = softmax with a sink over the cache          res32.window_attn (G = 1: all heads read the one cached row)
       a    = (o_c Wuv^T per head) * sigmoid(proj_g)      batched GEMM + res32.gate_mul
+      (bf16, cached rows wider than the portion kernel takes: prompt portions instead attend per head over keys
+       [Wuk c | rotated part] and values Wuv c up-projected from their sequences' cached rows into pages of their own,
+       res32.latent_expand_write; decode rows stay on the cached rows)
     retention layer:
       proj = h @ [Wq | Wk | Wv | Wg]^T                   ONE GEMM
       o    = S <- a_h S + k v^T, S^T q over the slot     res32.retention (rotation of q, k inside; state fp32 [H, D, Dv])
       a    = o / rms(o) per head * silu(proj_g)          res32.head_norm_gate
-    x     += norm1b(a @ Wo^T)                            res32.gated_norm_residual (no gate)
-    h2     = norm2(x)
+    x     += norm1b(a @ Wo^T);  h2 = norm2(x)            res32.gated_norm_residual (no gate; both norms in one pass)
     dense:   y = (glu_clamped(h2 @ [Wgate | Wup]^T)) @ Wdown^T             res32.glu
     experts: top-k of the router's logits + bias, softmax over the chosen  res32.router (fp32)
              y = sum_j s_j expert_j(h2) + shared(h2)                       res32.expert_rows / grouped GEMMs, moe_combine
-    x     += norm2b(y)
+    x     += norm2b(y);  h = the next run's norm1(x)     res32.gated_norm_residual
 
 ``cfg.runs`` lists the layer of every run: a looped span repeats in a row with the same weights, and every run has its
 own pages in the paged cache (attention) or its own matrix in the recurrent-state slots (retention).
