@@ -21,10 +21,10 @@ int r32_window_attn_mfma_ok(int, int);
 int r32_window_attn_mfma(const float*, const void*, const void*, long long, long long, int, const int*, const int*,
                          const int*, int, int, const int*, int, const float*, const float*, int, void*, int, int, int, int, int,
                          hipStream_t);
-int r32_window_attn_decode_ok(int, int);
+int r32_window_attn_decode_ok(int, int, int);
 int r32_window_attn_decode_splits(int, int, int, int, int);
 int r32_window_attn_decode(const float*, const void*, const void*, long long, long long, int, const int*, const int*, int,
-                           const float*, const float*, int, float*, float*, int, int, void*, int, int, int, int, int, int,
+                           const float*, const float*, int, float*, float*, int, int, void*, int, int, int, int, int, int, int,
                            hipStream_t);
 int r32_conv_hist(const void*, int, const float*, int, int, float*, long long, const int*, const int*, const int*,
                   const int*, void*, int, void*, int, int, int, int, int, int, int, hipStream_t);
@@ -243,7 +243,9 @@ void window_attn(Tensor q, Tensor k_cache, Tensor v_cache, Tensor positions, c10
 }
 
 bool window_attn_mfma_ok(int64_t D, int64_t Dv) { return r32_window_attn_mfma_ok((int)D, (int)Dv) != 0; }
-bool window_attn_decode_ok(int64_t D, int64_t Dv) { return r32_window_attn_decode_ok((int)D, (int)Dv) != 0; }
+bool window_attn_decode_ok(int64_t D, int64_t Dv, bool values_in_keys) {
+  return r32_window_attn_decode_ok((int)D, (int)Dv, values_in_keys ? 1 : 0) != 0;
+}
 
 const float* sink_ptr(const c10::optional<Tensor>& sink, int64_t H, const char* name) {
   if (!sink.has_value()) return nullptr;
@@ -292,7 +294,7 @@ void window_attn_mfma(Tensor q, Tensor k_cache, Tensor v_cache, Tensor positions
 // positions[b].  max_keys: a host-side upper bound of the keys a row sees (min(window, longest context)).
 void window_attn_decode(Tensor q, Tensor k_cache, Tensor v_cache, Tensor positions, Tensor block_tables,
                         c10::optional<Tensor> bias, int64_t window, int64_t max_keys, Tensor out, int64_t H, int64_t G,
-                        c10::optional<Tensor> sink) {
+                        c10::optional<Tensor> sink, bool values_in_keys) {
   want(q, torch::kFloat32, "window_attn_decode q");
   want(positions, torch::kInt32, "window_attn_decode positions");
   want(block_tables, torch::kInt32, "window_attn_decode block_tables");
@@ -305,7 +307,7 @@ void window_attn_decode(Tensor q, Tensor k_cache, Tensor v_cache, Tensor positio
   cache_layout(k_cache, v_cache, NB, BS, nk, nv, "window_attn_decode");
   TORCH_CHECK(G > 0 && H > 0 && H % G == 0 && nk % G == 0 && nv % G == 0, "window_attn_decode: head counts");
   const int D = nk / (int)G, Dv = nv / (int)G;
-  TORCH_CHECK(r32_window_attn_decode_ok(D, Dv), "window_attn_decode: sizes not built");
+  TORCH_CHECK(r32_window_attn_decode_ok(D, Dv, values_in_keys ? 1 : 0), "window_attn_decode: sizes not built");
   const int ldo = row_stride(out, "window_attn_decode out");
   TORCH_CHECK(k_cache.stride(0) % 8 == 0 && v_cache.stride(0) % 8 == 0 && ((uintptr_t)k_cache.data_ptr() & 15) == 0 &&
                   ((uintptr_t)v_cache.data_ptr() & 15) == 0, "window_attn_decode: cache alignment");
@@ -319,7 +321,8 @@ void window_attn_decode(Tensor q, Tensor k_cache, Tensor v_cache, Tensor positio
                               (long long)v_cache.stride(0), BS, positions.data_ptr<int>(), block_tables.data_ptr<int>(),
                               (int)block_tables.size(1), bias.has_value() ? bias->data_ptr<float>() : nullptr,
                               sink_ptr(sink, H, "window_attn_decode"), (int)window, po, po + (int64_t)B * H * S * Dv, S,
-                              (int)max_keys, out.data_ptr(), ldo, B, (int)H, (int)G, D, Dv, stream()), "window_attn_decode");
+                              (int)max_keys, out.data_ptr(), ldo, B, (int)H, (int)G, D, Dv, values_in_keys ? 1 : 0, stream()),
+       "window_attn_decode");
 }
 
 

@@ -2,13 +2,15 @@
 // instantiation is compiled in a file of its own, wattn_decode_wide.hip, with its own code generation flags).
 #include "wattn_decode_kernel.h"
 
-// Sizes the decode kernel is built for.
-extern "C" int r32_window_attn_decode_ok(int D, int Dv) {
+// Sizes the decode kernel is built for.  vk: the caller's value pages repeat the first Dv entries of the key rows (a
+// latent that is key and value at once); only then does the wide kernel apply (it reads its values from the key rows).
+extern "C" int r32_window_attn_decode_ok(int D, int Dv, int vk) {
   const bool small = (D == 32 || D == 64 || D == 128) && (Dv == 32 || Dv == 64 || Dv == 128);
-  return small || (D == 576 && Dv == 512);
+  return small || (vk && D == 576 && Dv == 512);
 }
 
-extern "C" int r32_window_attn_decode_wide_launch(const WAttnDecodeParams* p, int gx, int gy, int gz, hipStream_t s);
+extern "C" int r32_window_attn_decode_wide_launch(const WAttnDecodeParams* p, int gx, int gy, int gz, int chunks_per_group,
+                                                  hipStream_t s);
 
 // out[b, h, :] = sum_s exp(m_s - M) o_s / sum_s exp(m_s - M) l_s  (splits that saw no key have l = 0)
 // sink (or null): exp(sink_h) joins the denominator.
@@ -47,11 +49,13 @@ int launch_decode_nv(const WAttnDecodeParams& p, int nv, dim3 grid, hipStream_t 
 // Splits for a decode step of B sequences whose windows hold at most max_keys keys: about 2048 waves (two per SIMD),
 // at least 64 keys each.  Measured at 64 sequences x 8 kv heads x 2048 keys of 128: 3 splits 150 us, 4 splits
 // (2048 waves) 130 us, 8 splits 155 us, 16 splits 146 us (shorter key runs per wave, larger partials to merge).
-// Wide rows (D = 576): workgroups of four waves, about 1024 of them, at least 128 keys each (their partials are large).
+// Wide rows (D = 576): workgroups of four or eight waves, about 512 of them, at least 128 keys each (their partials
+// are large).
 extern "C" int r32_window_attn_decode_splits(int B, int G, int Hg, int max_keys, int D) {
-  const int waves = B * G * ((Hg + 15) / 16);
   const bool wide = D > 128;
-  int s = ((wide ? 1024 : 2048) + waves - 1) / waves;
+  const int chunks = (Hg + 15) / 16;
+  const int waves = B * G * (wide && chunks > 1 ? (chunks + 1) / 2 : chunks);  // wide rows: workgroups
+  int s = ((wide ? 512 : 2048) + waves - 1) / waves;
   const int by_keys = wide ? (max_keys + 32 + 127) / 128 : (max_keys + 32 + 63) / 64;
   if (s > by_keys) s = by_keys;
   if (s > 64) s = 64;
@@ -64,9 +68,9 @@ extern "C" int r32_window_attn_decode(const float* q, const void* k_cache, const
                                       long long vb_stride, int block_size, const int* positions, const int* block_tables,
                                       int bt_width, const float* bias, const float* sink, int window, float* part_o,
                                       float* part_ml, int S, int max_keys, void* out, int ldo, int B, int H, int G, int D,
-                                      int Dv, hipStream_t s) {
+                                      int Dv, int vk, hipStream_t s) {
   if (B <= 0) return 0;
-  if (!r32_window_attn_decode_ok(D, Dv) || H % G != 0 || S < 1 || (block_size & (block_size - 1)) != 0) return -1;
+  if (!r32_window_attn_decode_ok(D, Dv, vk) || H % G != 0 || S < 1 || (block_size & (block_size - 1)) != 0) return -1;
   WAttnDecodeParams p;
   p.q = q; p.k_cache = (const bf16_t*)k_cache; p.v_cache = (const bf16_t*)v_cache; p.kb_stride = kb_stride;
   p.vb_stride = vb_stride; p.block_size = block_size; p.positions = positions; p.block_tables = block_tables;
@@ -81,7 +85,8 @@ extern "C" int r32_window_attn_decode(const float* q, const void* k_cache, const
   const dim3 grid(B, G * ((Hg + 15) / 16), S);
   int rc = -1;
   if (D == 576 && Dv == 512) {  // one wide row for all heads: a low-rank attention's cached latent + rotated part
-    rc = r32_window_attn_decode_wide_launch(&p, (int)grid.x, (int)grid.y, (int)grid.z, s);
+    const int chunks = (Hg + 15) / 16, nc = chunks > 1 ? 2 : 1;  // more than 16 heads: two chunks per workgroup
+    rc = r32_window_attn_decode_wide_launch(&p, B, G * ((chunks + nc - 1) / nc), S, nc, s);
   } else {
     switch (D / 32) {
       case 1: rc = launch_decode_nv<1>(p, Dv / 16, grid, s); break;

@@ -39,17 +39,21 @@ struct WAttnDecodeParams {
 // owns NV / NW of the 16-column value tiles (wide value rows: the accumulators of one wave would leave no registers
 // for loads in flight).  With NW > 1 a tile's 32 key rows go through LDS once for all the waves (fetched into registers
 // one tile ahead); a wave's own value words still come straight from the cache.  QLO = false: q enters as its bf16
-// rounding only (one MFMA per operand instead of two).
-template <int ND, int NV, int NW = 1, bool QLO = true>
-__global__ void __launch_bounds__(64 * NW) window_attn_decode_kernel(const WAttnDecodeParams p) {
-  constexpr int D = 32 * ND, DV = 16 * NV, NVW = NV / NW;
+// rounding only (one MFMA per operand instead of two).  VK = true (with NW > 1): the values ARE the first DV entries of
+// the key rows (a cached latent that is key and value at once), so the value operands are gathered from the staged
+// rows in LDS and the value pages are not read at all.
+template <int ND, int NV, int NW = 1, bool QLO = true, bool VK = false, int NC = 1>
+__global__ void __launch_bounds__(64 * NW * NC) window_attn_decode_kernel(const WAttnDecodeParams p) {
+  constexpr int D = 32 * ND, DV = 16 * NV, NVW = NV / NW, NT = 64 * NW * NC;  // NT: threads of the workgroup
   static_assert(NV % NW == 0, "value tiles divide among the waves");
   const int b = blockIdx.x, split = blockIdx.z;
   const int H = p.H, G = p.G, Hg = H / G, chunks = (Hg + 15) / 16;
-  const int g = blockIdx.y / chunks, h0 = g * Hg + (blockIdx.y % chunks) * 16;
-  const int nh = min(16, g * Hg + Hg - h0);  // heads of this chunk
   // (one wave: the wave index is a compile-time zero, so the value tiles' offsets stay immediates)
-  const int lane = NW > 1 ? (int)(threadIdx.x & 63) : (int)threadIdx.x, wv = NW > 1 ? (int)(threadIdx.x >> 6) : 0;
+  const int lane = NT > 64 ? (int)(threadIdx.x & 63) : (int)threadIdx.x, wv_all = NT > 64 ? (int)(threadIdx.x >> 6) : 0;
+  const int wv = NC > 1 ? wv_all % NW : wv_all, cw = NC > 1 ? wv_all / NW : 0;
+  const int cgroups = (chunks + NC - 1) / NC;  // workgroups per kv head
+  const int g = blockIdx.y / cgroups, h0 = g * Hg + ((blockIdx.y % cgroups) * NC + cw) * 16;
+  const int nh = min(16, g * Hg + Hg - h0);  // heads of this chunk (<= 0: a wave past the last chunk only helps staging)
   const int r16 = lane & 15, g4 = lane >> 4;
   const int i = p.positions[b];
   const int j_lo = max(0, i - p.window + 1);
@@ -89,15 +93,15 @@ __global__ void __launch_bounds__(64 * NW) window_attn_decode_kernel(const WAttn
 
   constexpr bool kStage = NW > 1;
   constexpr int KLD = D + 8;                                       // LDS row stride: rows start in different banks
-  constexpr int KCH = (32 * (D / 8) + 64 * NW - 1) / (64 * NW);    // 16-byte words per thread and tile
+  constexpr int KCH = (32 * (D / 8) + NT - 1) / NT;                 // 16-byte words per thread and tile
   __shared__ __attribute__((aligned(16))) bf16_t K_s[kStage ? 32 * KLD : 8];
   uint4v kreg[kStage ? KCH : 1];
   auto fetch = [&](int t0) {
 #pragma unroll
     for (int u = 0; u < KCH; ++u) {
-      const int c = (int)threadIdx.x + 64 * NW * u;
+      const int c = min((int)threadIdx.x + NT * u, 32 * (D / 8) - 1);
       const int key = c / (D / 8), dc = c % (D / 8);
-      const int j = min(t0 + min(key, 31), i);  // (rows past the token are masked below: any valid row does)
+      const int j = min(t0 + key, i);  // (rows past the token are masked below: any valid row does)
       kreg[u] = *reinterpret_cast<const uint4v*>(p.k_cache + (long long)page_of(j) * p.kb_stride +
                                                  ((long long)page_off(j) * G + g) * D + dc * 8);
     }
@@ -105,7 +109,7 @@ __global__ void __launch_bounds__(64 * NW) window_attn_decode_kernel(const WAttn
   auto stash = [&]() {
 #pragma unroll
     for (int u = 0; u < KCH; ++u) {
-      const int c = (int)threadIdx.x + 64 * NW * u;
+      const int c = (int)threadIdx.x + NT * u;
       if (c < 32 * (D / 8)) *reinterpret_cast<uint4v*>(&K_s[(c / (D / 8)) * KLD + (c % (D / 8)) * 8]) = kreg[u];
     }
   };
@@ -183,9 +187,19 @@ __global__ void __launch_bounds__(64 * NW) window_attn_decode_kernel(const WAttn
     for (int n = 0; n < NVW; ++n) {
 #pragma unroll
       for (int r = 0; r < 4; ++r) O[n][r] *= ar[r];
-      const short4v b0 = *reinterpret_cast<const short4v*>(va + 64 * (wv * NVW + n));
-      const short4v b1 = *reinterpret_cast<const short4v*>(vb + 64 * (wv * NVW + n));
-      const short8 bb = short8{b0[0], b0[1], b0[2], b0[3], b1[0], b1[1], b1[2], b1[3]};
+      short8 bb;
+      if (kStage && VK) {
+        const bf16_t* col = &K_s[(4 * g4) * KLD + 16 * (wv * NVW + n) + r16];  // this lane's value column, key 4 g4
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          bb[e] = (short)col[e * KLD];
+          bb[4 + e] = (short)col[(16 + e) * KLD];
+        }
+      } else {
+        const short4v b0 = *reinterpret_cast<const short4v*>(va + 64 * (wv * NVW + n));
+        const short4v b1 = *reinterpret_cast<const short4v*>(vb + 64 * (wv * NVW + n));
+        bb = short8{b0[0], b0[1], b0[2], b0[3], b1[0], b1[1], b1[2], b1[3]};
+      }
       O[n] = mfma16(ph, bb, O[n]);
       O[n] = mfma16(pl, bb, O[n]);
     }

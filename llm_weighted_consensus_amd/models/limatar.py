@@ -356,7 +356,7 @@ class LimatarModel:
             oc = torch.empty(n_abs, H * Cv, dtype=dt, device=self.device)
             if n_dec:
                 res32.window_attn(qf[:n_dec], kc, vc, pa[:n_dec], plan.dec_tables, z, z, UNBOUNDED, oc[:n_dec], H, 1,
-                                  cores=True, sink=x["sink"])
+                                  cores=True, sink=x["sink"], values_in_keys=True)
             if n_abs > n_dec:
                 ch = plan.chunk
                 res32.window_attn(qf[n_dec:], kc, vc, pa[n_dec:], ch["block_tables"], z, z, UNBOUNDED, oc[n_dec:], H, 1,

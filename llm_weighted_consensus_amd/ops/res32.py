@@ -105,22 +105,25 @@ def window_attn(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, p
                 block_tables: torch.Tensor, r1: torch.Tensor, r2: torch.Tensor, window: int, out: torch.Tensor,
                 H: int, G: int, cu_q: Optional[torch.Tensor] = None, k_lens: Optional[torch.Tensor] = None,
                 max_q: int = 0, bias: Optional[torch.Tensor] = None, cores: Optional[bool] = None,
-                sink: Optional[torch.Tensor] = None) -> torch.Tensor:
+                sink: Optional[torch.Tensor] = None, values_in_keys: bool = False) -> torch.Tensor:
     """Sliding-window attention over the paged cache with the bias -r1_h ln(1 + r2_h (i - j)); ``q`` fp32
     [T, H*D] pre-scaled; row t reads table row t (``cu_q`` None) or the item whose ``cu_q`` range holds t.
     Over a bf16 cache whose sizes the matrix-core kernels are built for, prompt portions run on the portion kernel
     (it wants ``k_lens``, ``max_q`` and the ``bias`` table of :func:`distance_bias`) and decode rows on the
     split-key decode kernel (``bias``); everything else on the general kernel.  ``cores=True`` with ``bias`` None:
     the matrix-core kernels without a distance bias (r1 = 0: plain causal or windowed softmax attention).
-    ``sink`` (fp32 [H]): exp(sink_h) joins head h's softmax denominator; it has no key and no value."""
+    ``sink`` (fp32 [H]): exp(sink_h) joins head h's softmax denominator; it has no key and no value.
+    ``values_in_keys``: the caller guarantees that every token's value row repeats the first Dv entries of its key row
+    (a cached latent that is key and value at once); the decode kernel for one wide row (576 / 512) then takes its
+    values from the key rows."""
     K = kernels()
     bs = k_cache.shape[1]
     D, Dv = k_cache.shape[2] // G, v_cache.shape[2] // G
     cores = (bias is not None or bool(cores)) and k_cache.dtype == torch.bfloat16 and bs & (bs - 1) == 0
-    if cores and cu_q is None and positions.numel() > 0 and K.window_attn_decode_ok(D, Dv):
+    if cores and cu_q is None and positions.numel() > 0 and K.window_attn_decode_ok(D, Dv, bool(values_in_keys)):
         max_keys = min(int(window), block_tables.shape[1] * k_cache.shape[1])
         K.window_attn_decode(q, k_cache, v_cache, positions, block_tables, bias, int(window), max_keys, out, int(H), int(G),
-                             sink)
+                             sink, bool(values_in_keys))
         return out
     if cores and cu_q is not None and k_lens is not None and max_q > 0 and K.window_attn_mfma_ok(D, Dv):
         K.window_attn_mfma(q, k_cache, v_cache, positions, cu_q, k_lens, int(max_q), block_tables, bias, int(window), out,
