@@ -84,7 +84,7 @@ def _limatar(size: dict, layers: int, device, seed: int, experts: int = 8, top: 
     dense = {"kind": "dense", "ff": size["ffn"], "limit": 7.0}
     lat = {"heads": H, "dim": D, "rot_dim": D // 2, "vdim": D, "q_rank": 3 * d // 8, "kv_rank": 4 * D, "scale": (D + D // 2) ** -0.5,
            "rot": {"base": 10000.0, "dims": D // 2, "scaling": {"factor": 4.0, "original": 1024, "fast": 32.0, "slow": 1.0}}}
-    ret = {"heads": H, "dim": D, "vdim": D, "decay": [1.0 - 2.0 ** (-5 - 3 * h / max(H - 1, 1)) for h in range(H)],
+    ret = {"heads": H, "dim": D, "vdim": D, "decay": [1.0 - 2.0 ** (-4 - 4 * h / max(H - 1, 1)) for h in range(H)],
            "rot": {"base": 10000.0, "dims": D}}
     specs = []
     for i in range(layers):
