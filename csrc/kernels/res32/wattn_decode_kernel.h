@@ -35,8 +35,8 @@ struct WAttnDecodeParams {
   int H, G, S, keys_per_split;  // keys_per_split: a multiple of 32
 };
 
-// NW waves per workgroup share one (sequence, head chunk, split): every wave forms the scores of all keys itself and
-// owns NV / NW of the 16-column value tiles (wide value rows: the accumulators of one wave would leave no registers
+// NW waves per workgroup share one (sequence, head chunk, split): the waves form the scores of a tile's keys together
+// (NW = 4: each a quarter of the MFMAs, the partial scores meet in LDS) and each owns NV / NW of the 16-column value tiles (wide value rows: the accumulators of one wave would leave no registers
 // for loads in flight).  With NW > 1 a tile's 32 key rows go through LDS once for all the waves (fetched into registers
 // one tile ahead); a wave's own value words still come straight from the cache.  QLO = false: q enters as its bf16
 // rounding only (one MFMA per operand instead of two).  VK = true (with NW > 1): the values ARE the first DV entries of
@@ -73,13 +73,19 @@ __global__ void __launch_bounds__(64 * NW * NC) window_attn_decode_kernel(const 
   const bool h_valid = r16 < nh;
   const int h = h0 + (h_valid ? r16 : 0);
 
-  short8 qhi[ND], qlo[QLO ? ND : 1];
+  // With NW = 4 staged waves the scores of a tile are formed ONCE per chunk: wave w multiplies key subtile (w & 1) with
+  // half (w >> 1) of the row's 32-entry slices, the halves meet through LDS.  Such a wave keeps only its half of q.
+  constexpr bool kSplitQK = NW == 4;
+  static_assert(!kSplitQK || ND % 2 == 0, "the slices divide into two halves");
+  constexpr int NDW = kSplitQK ? ND / 2 : ND;
+  const int kd0 = kSplitQK ? (wv >> 1) * NDW : 0;
+  short8 qhi[NDW], qlo[QLO ? NDW : 1];
 #pragma unroll
-  for (int kd = 0; kd < ND; ++kd) {
+  for (int kd = 0; kd < NDW; ++kd) {
 #pragma unroll
     for (int e = 0; e < 8; ++e) {
       float x = 0.f;
-      if (h_valid) x = p.q[((size_t)b * H + h) * D + kd * 32 + 8 * g4 + e];
+      if (h_valid) x = p.q[((size_t)b * H + h) * D + (kd0 + kd) * 32 + 8 * g4 + e];
       const bf16_t hi = f2bf(x);
       qhi[kd][e] = (short)hi;
       if (QLO) qlo[kd][e] = (short)f2bf(x - bf2f(hi));
@@ -95,6 +101,7 @@ __global__ void __launch_bounds__(64 * NW * NC) window_attn_decode_kernel(const 
   constexpr int KLD = D + 8;                                       // LDS row stride: rows start in different banks
   constexpr int KCH = (32 * (D / 8) + NT - 1) / NT;                 // 16-byte words per thread and tile
   __shared__ __attribute__((aligned(16))) bf16_t K_s[kStage ? 32 * KLD : 8];
+  __shared__ __attribute__((aligned(16))) float4v S_x[NW == 4 ? NC * NW * 64 : 1];  // partial scores of the waves
   uint4v kreg[kStage ? KCH : 1];
   auto fetch = [&](int t0) {
 #pragma unroll
@@ -122,6 +129,20 @@ __global__ void __launch_bounds__(64 * NW * NC) window_attn_decode_kernel(const 
   for (int t0 = base; t0 <= last; t0 += 32) {  // (base and last are the same for every wave of the workgroup)
     if (kStage && t0 + 32 <= last) fetch(t0 + 32);
     float4v sacc[2];
+    if constexpr (kSplitQK) {
+      float4v part = float4v{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+      for (int kd = 0; kd < NDW; ++kd) {
+        const short8 a = *reinterpret_cast<const short8*>(&K_s[((wv & 1) * 16 + r16) * KLD + (kd0 + kd) * 32 + 8 * g4]);
+        part = mfma16(a, qhi[kd], part);
+        if (QLO) part = mfma16(a, qlo[kd], part);
+      }
+      S_x[(cw * NW + wv) * 64 + lane] = part;
+      __syncthreads();  // (the barriers at the tile's end keep the next tile's partials from overtaking these reads)
+#pragma unroll
+      for (int sub = 0; sub < 2; ++sub)
+        sacc[sub] = S_x[(cw * NW + sub) * 64 + lane] + S_x[(cw * NW + sub + 2) * 64 + lane];
+    } else {
 #pragma unroll
     for (int sub = 0; sub < 2; ++sub) {
       sacc[sub] = float4v{0.f, 0.f, 0.f, 0.f};
@@ -143,6 +164,7 @@ __global__ void __launch_bounds__(64 * NW * NC) window_attn_decode_kernel(const 
         }
       }
     }
+    }  // (scores without the split)
     float s[8];
     bool ok[8];
     float mx = -1e30f;
