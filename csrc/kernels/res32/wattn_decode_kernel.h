@@ -35,13 +35,16 @@ struct WAttnDecodeParams {
   int H, G, S, keys_per_split;  // keys_per_split: a multiple of 32
 };
 
-// NW waves per workgroup share one (sequence, head chunk, split): the waves form the scores of a tile's keys together
-// (NW = 4: each a quarter of the MFMAs, the partial scores meet in LDS) and each owns NV / NW of the 16-column value tiles (wide value rows: the accumulators of one wave would leave no registers
-// for loads in flight).  With NW > 1 a tile's 32 key rows go through LDS once for all the waves (fetched into registers
-// one tile ahead); a wave's own value words still come straight from the cache.  QLO = false: q enters as its bf16
-// rounding only (one MFMA per operand instead of two).  VK = true (with NW > 1): the values ARE the first DV entries of
-// the key rows (a cached latent that is key and value at once), so the value operands are gathered from the staged
-// rows in LDS and the value pages are not read at all.
+// NW waves per workgroup share one (sequence, head chunk, split).  With NW > 1 a tile's 32 key rows go through LDS
+// once for all the waves (fetched into registers one tile ahead), and each wave owns NV / NW of the 16-column value
+// tiles (wide value rows: the accumulators of one wave would leave no registers for loads in flight).  NW = 4: the
+// waves also form the tile's scores together, each a quarter of the MFMAs (one key subtile times half of the row's
+// 32-entry slices), and the partial scores meet in LDS.
+// QLO = false: q enters as its bf16 rounding only (one MFMA per operand instead of two).
+// VK = true (with NW > 1): the values ARE the first DV entries of the key rows (a cached latent that is key and value
+// at once), so the value operands are gathered from the staged rows in LDS and the value pages are not read at all.
+// NC > 1: NC head chunks (16 heads each) of one kv head share the workgroup and with it every staged key row (waves
+// [c NW, (c + 1) NW) serve chunk c).
 template <int ND, int NV, int NW = 1, bool QLO = true, bool VK = false, int NC = 1>
 __global__ void __launch_bounds__(64 * NW * NC) window_attn_decode_kernel(const WAttnDecodeParams p) {
   constexpr int D = 32 * ND, DV = 16 * NV, NVW = NV / NW, NT = 64 * NW * NC;  // NT: threads of the workgroup
