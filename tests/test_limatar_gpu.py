@@ -130,7 +130,7 @@ def _paged(n_tokens, bs, nk, nv, dtype, gpu, seed=0):
 
 
 @pytest.mark.parametrize("dtype,tol", [(torch.float32, 2e-5), (torch.bfloat16, 2e-2)])
-@pytest.mark.parametrize("H,D,Dv", [(3, 40, 24), (7, 120, 88), (2, 328, 320), (1, 8, 8), (4, 128, 128), (5, 64, 32), (3, 192, 128),
+@pytest.mark.parametrize("H,D,Dv", [(3, 40, 24), (7, 120, 88), (2, 328, 320), (1, 8, 8), (4, 128, 128), (5, 64, 32), (20, 64, 32), (3, 192, 128),
                                     (17, 576, 512)])
 def test_softmax_with_sinks_over_one_shared_row(gpu, dtype, tol, H, D, Dv):
     """All heads read ONE cached row per token (G = 1); exp(sink_h) joins the denominator.  Decode rows and a prompt
