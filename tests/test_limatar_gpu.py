@@ -350,6 +350,10 @@ def _configs():
     # a latent wide enough for the 576 / 512 decode kernel (17 heads: two head chunks)
     out["deep"] = dict(width=64, vocab=200, loop=None, layers=[
         O.latent_layer(17, 16, 64, 16, 24, 320, O.dense(64)), O.retention_layer(2, 16, 16, None)])
+    # a width that is no multiple of four (the kernels' one-element paths), 20 heads (two head chunks of the decode kernel),
+    # 33 router outputs (the wave-wide router), a retention head wider than 128, the whole model looped
+    out["ragged"] = dict(width=50, vocab=97, loop=(0, 2, 2), layers=[
+        O.latent_layer(20, 6, 4, 5, 11, 26, O.moe(33, 4, 10)), O.retention_layer(2, 136, 20, O.dense(30, limit=2.0), rot_dims=100)])
     # the same layers with two passes of the span: bf16 comparisons (rounding differences grow with every pass of the
     # same weights, and a routing choice flipped by rounding changes a whole row)
     out["mixed2"] = {**out["mixed"], "loop": (1, 3, 2)}
@@ -406,7 +410,7 @@ def _err(got, ref, dtype=torch.float32):
 TOL = {torch.float32: 3e-4, torch.bfloat16: 0.5}
 
 
-@pytest.mark.parametrize("name,dtype", [(n, d) for d in (torch.float32, torch.bfloat16) for n in ("mixed", "odd", "recurrent", "attentive", "wide", "deep")
+@pytest.mark.parametrize("name,dtype", [(n, d) for d in (torch.float32, torch.bfloat16) for n in ("mixed", "odd", "recurrent", "attentive", "wide", "deep", "ragged")
                                         if (n, d) != ("mixed", torch.bfloat16)] + [("mixed2", torch.bfloat16)])
 def test_whole_prompt_and_layer_runs(gpu, tmp_path, name, dtype):
     """A whole prompt in one step: the stream after every layer RUN (looped layers count each time) and the logits."""
@@ -454,7 +458,7 @@ def test_few_wanted_rows_and_what_they_leave(gpu, tmp_path, name, dtype):
 
 @pytest.mark.parametrize("name,dtype", [("mixed", torch.float32), ("odd", torch.float32), ("recurrent", torch.float32),
                                         ("attentive", torch.bfloat16), ("mixed2", torch.bfloat16), ("wide", torch.bfloat16),
-                                        ("deep", torch.bfloat16)])
+                                        ("deep", torch.bfloat16), ("ragged", torch.float32), ("ragged", torch.bfloat16)])
 def test_decode_token_by_token_and_portions(gpu, tmp_path, name, dtype):
     """The same logits whether a prompt comes whole, token by token from the first token on, or in portions of
     changing sizes (down to two tokens; cut inside pages and inside the recurrence kernel's tiles)."""
