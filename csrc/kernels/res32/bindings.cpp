@@ -15,16 +15,16 @@ int r32_xielu(const void*, int, const void*, void*, int, int, int, int, hipStrea
 int r32_residual_add_scaled(float*, const void*, float, long long, int, hipStream_t);
 int r32_residual_add_partials(float*, const float*, int, float, long long, hipStream_t);
 int r32_window_attn(const float*, const void*, const void*, long long, long long, int, const int*, const int*, int,
-                    const int*, int, const float*, const float*, const float*, int, void*, int, int, int, int, int, int, int,
+                    const int*, int, const float*, const float*, const float*, int, int, void*, int, int, int, int, int, int, int,
                     hipStream_t);
 int r32_window_attn_mfma_ok(int, int);
 int r32_window_attn_mfma(const float*, const void*, const void*, long long, long long, int, const int*, const int*,
-                         const int*, int, int, const int*, int, const float*, const float*, int, void*, int, int, int, int, int,
+                         const int*, int, int, const int*, int, const float*, const float*, int, int, void*, int, int, int, int, int,
                          hipStream_t);
 int r32_window_attn_decode_ok(int, int, int);
 int r32_window_attn_decode_splits(int, int, int, int, int);
 int r32_window_attn_decode(const float*, const void*, const void*, long long, long long, int, const int*, const int*, int,
-                           const float*, const float*, int, float*, float*, int, int, void*, int, int, int, int, int, int, int,
+                           const float*, const float*, int, int, float*, float*, int, int, void*, int, int, int, int, int, int, int,
                            hipStream_t);
 int r32_conv_hist(const void*, int, const float*, int, int, float*, long long, const int*, const int*, const int*,
                   const int*, void*, int, void*, int, int, int, int, int, int, int, hipStream_t);
@@ -34,7 +34,7 @@ int r32_delta_rule(float*, int, const void*, int, int, int, const float*, const 
                    const int*, const int*, float*, int, int, int, int, int, int, int, int, hipStream_t);
 int r32_head_norm_gate(const float*, int, const void*, int, const float*, void*, int, int, int, int, float, int, int,
                        hipStream_t);
-int r32_embed_rows(const void*, const int*, float*, int, int, int, int, hipStream_t);
+int r32_embed_rows(const void*, const int*, float*, int, int, int, float, int, hipStream_t);
 int r32_head_norm_kv_write(const void*, int, int, int, const int*, const int*, float*, void*, void*, long long, long long,
                            int, int, int, int, int, int, float, float, float, int, int, hipStream_t);
 int r32_gate_mul(void*, int, const void*, int, int, int, int, int, hipStream_t);
@@ -63,6 +63,17 @@ int r32_retention_prep(const void*, int, int, const float*, float, const int*, f
 int r32_retention(const float*, const void*, int, const float*, float*, long long, const int*, const int*, const int*, float*,
                   int, int, int, int, int, int, hipStream_t);
 int r32_glu(const void*, int, void*, int, int, int, int, float, float, int, hipStream_t);
+int r32_gelu(const void*, int, void*, int, int, int, int, hipStream_t);
+int r32_rot_kv_write(const void*, int, const float*, const float*, const float*, float, int, const float*, const int*,
+                     const int*, float*, void*, void*, long long, long long, int, int, int, int, int, int, float, float, int,
+                     hipStream_t);
+int r32_head_gate_unrotate(const void*, int, const void*, int, const float*, const int*, void*, int, int, int, int, float,
+                           int, hipStream_t);
+int r32_add_rmsnorm(float*, const void*, int, const float*, void*, int, int, int, float, int, hipStream_t);
+int r32_chan_rule_max_dim();
+int r32_chan_rule(const void*, int, int, float*, int, const void*, int, int, const float*, const float*, float, const void*,
+                  int, int, float*, float*, float*, long long, const int*, const int*, const int*, float*, int, int, int, int,
+                  int, int, int, int, int, hipStream_t);
 }
 
 namespace {
@@ -204,7 +215,7 @@ void residual_add_partials(Tensor x, Tensor parts, double m) {
 // sink: fp32 [H], exp(sink_h) joins head h's softmax denominator (no key, no value), or absent.
 void window_attn(Tensor q, Tensor k_cache, Tensor v_cache, Tensor positions, c10::optional<Tensor> cu_q,
                  Tensor block_tables, Tensor r1, Tensor r2, int64_t window, Tensor out, int64_t H, int64_t G,
-                 c10::optional<Tensor> sink) {
+                 c10::optional<Tensor> sink, int64_t chunk) {
   want(q, torch::kFloat32, "window_attn q");
   const int f = act_f32(k_cache, "window_attn k_cache");
   want(positions, torch::kInt32, "window_attn positions");
@@ -238,7 +249,7 @@ void window_attn(Tensor q, Tensor k_cache, Tensor v_cache, Tensor positions, c10
   }
   done(r32_window_attn(q.data_ptr<float>(), k_cache.data_ptr(), v_cache.data_ptr(), (long long)k_cache.stride(0),
                        (long long)v_cache.stride(0), BS, positions.data_ptr<int>(), cu, items, block_tables.data_ptr<int>(),
-                       width, r1.data_ptr<float>(), r2.data_ptr<float>(), sk, (int)window, out.data_ptr(), ldo, T, (int)H, (int)G,
+                       width, r1.data_ptr<float>(), r2.data_ptr<float>(), sk, (int)window, (int)chunk, out.data_ptr(), ldo, T, (int)H, (int)G,
                        D, Dv, f, stream()), "window_attn");
 }
 
@@ -259,7 +270,7 @@ const float* sink_ptr(const c10::optional<Tensor>& sink, int64_t H, const char* 
 // Positions ascend by one along each item's rows.
 void window_attn_mfma(Tensor q, Tensor k_cache, Tensor v_cache, Tensor positions, Tensor cu_q, Tensor k_lens,
                       int64_t max_q, Tensor block_tables, c10::optional<Tensor> bias, int64_t window, Tensor out, int64_t H,
-                      int64_t G, c10::optional<Tensor> sink) {
+                      int64_t G, c10::optional<Tensor> sink, int64_t chunk) {
   want(q, torch::kFloat32, "window_attn_mfma q");
   want(positions, torch::kInt32, "window_attn_mfma positions");
   want(block_tables, torch::kInt32, "window_attn_mfma block_tables");
@@ -286,7 +297,7 @@ void window_attn_mfma(Tensor q, Tensor k_cache, Tensor v_cache, Tensor positions
                             (long long)v_cache.stride(0), BS, positions.data_ptr<int>(), cu_q.data_ptr<int>(),
                             k_lens.data_ptr<int>(), items, (int)max_q, block_tables.data_ptr<int>(),
                             (int)block_tables.size(1), bias.has_value() ? bias->data_ptr<float>() : nullptr,
-                            sink_ptr(sink, H, "window_attn_mfma"), (int)window, out.data_ptr(), ldo, (int)H, (int)G, D, Dv,
+                            sink_ptr(sink, H, "window_attn_mfma"), (int)window, (int)chunk, out.data_ptr(), ldo, (int)H, (int)G, D, Dv,
                             stream()), "window_attn_mfma");
 }
 
@@ -294,7 +305,7 @@ void window_attn_mfma(Tensor q, Tensor k_cache, Tensor v_cache, Tensor positions
 // positions[b].  max_keys: a host-side upper bound of the keys a row sees (min(window, longest context)).
 void window_attn_decode(Tensor q, Tensor k_cache, Tensor v_cache, Tensor positions, Tensor block_tables,
                         c10::optional<Tensor> bias, int64_t window, int64_t max_keys, Tensor out, int64_t H, int64_t G,
-                        c10::optional<Tensor> sink, bool values_in_keys) {
+                        c10::optional<Tensor> sink, bool values_in_keys, int64_t chunk) {
   want(q, torch::kFloat32, "window_attn_decode q");
   want(positions, torch::kInt32, "window_attn_decode positions");
   want(block_tables, torch::kInt32, "window_attn_decode block_tables");
@@ -320,7 +331,7 @@ void window_attn_decode(Tensor q, Tensor k_cache, Tensor v_cache, Tensor positio
   done(r32_window_attn_decode(q.data_ptr<float>(), k_cache.data_ptr(), v_cache.data_ptr(), (long long)k_cache.stride(0),
                               (long long)v_cache.stride(0), BS, positions.data_ptr<int>(), block_tables.data_ptr<int>(),
                               (int)block_tables.size(1), bias.has_value() ? bias->data_ptr<float>() : nullptr,
-                              sink_ptr(sink, H, "window_attn_decode"), (int)window, po, po + (int64_t)B * H * S * Dv, S,
+                              sink_ptr(sink, H, "window_attn_decode"), (int)window, (int)chunk, po, po + (int64_t)B * H * S * Dv, S,
                               (int)max_keys, out.data_ptr(), ldo, B, (int)H, (int)G, D, Dv, values_in_keys ? 1 : 0, stream()),
        "window_attn_decode");
 }
@@ -352,7 +363,8 @@ long long hist_layout(const Tensor& hist, int taps, int C, const char* name) {
   return (long long)hist.stride(0);
 }
 
-// mode 0: out = x + conv(x), out2 (optional) = x in out's dtype; mode 1: out = silu(conv(x)).  w fp32 [C, taps].
+// mode 0: out = x + conv(x), out2 (optional) = x in out's dtype; mode 1: out = silu(conv(x)); mode 2: out = conv(x).
+// w fp32 [C, taps].
 // advance: every item is ONE row (a decode step) and the kernel also moves the slots' histories on.
 void conv_hist(Tensor x, Tensor w, Tensor hist, Tensor row_item, Tensor cu, Tensor item_slot, Tensor positions, Tensor out,
                c10::optional<Tensor> out2, int64_t mode, bool advance) {
@@ -450,15 +462,15 @@ void head_norm_gate(Tensor o, c10::optional<Tensor> gate, c10::optional<Tensor> 
                           stream()), "head_norm_gate");
 }
 
-void embed_rows(Tensor table, Tensor tokens, Tensor out) {
+void embed_rows(Tensor table, Tensor tokens, Tensor out, double scale) {
   const int f = act_f32(table, "embed_rows table");
   TORCH_CHECK(table.dim() == 2 && table.is_contiguous(), "embed_rows: table [V, d]");
   want(tokens, torch::kInt32, "embed_rows tokens");
   want(out, torch::kFloat32, "embed_rows out");
   const int T = (int)tokens.numel(), d = (int)table.size(1);
   TORCH_CHECK(out.numel() == (int64_t)T * d, "embed_rows: out [T, d]");
-  done(r32_embed_rows(table.data_ptr(), tokens.data_ptr<int>(), out.data_ptr<float>(), T, d, (int)table.size(0), f, stream()),
-       "embed_rows");
+  done(r32_embed_rows(table.data_ptr(), tokens.data_ptr<int>(), out.data_ptr<float>(), T, d, (int)table.size(0), (float)scale, f,
+                      stream()), "embed_rows");
 }
 
 // proj [T, ...] row-dense: q at column 0 (H*D), k at k_off (G*D), values at v_off (G*Dv; v_off == k_off: the keys as
@@ -765,6 +777,133 @@ void glu(Tensor in, Tensor out, int64_t mode, double alpha, double limit) {
                f, stream()), "glu");
 }
 
+// out = z / 2 (1 + erf(z / sqrt 2)) over row-dense views of one dtype
+void gelu(Tensor in, Tensor out) {
+  const int f = act_f32(in, "gelu in");
+  const int ldi = row_stride(in, "gelu in"), ldo = row_stride(out, "gelu out");
+  TORCH_CHECK(out.is_cuda() && out.scalar_type() == in.scalar_type() && out.size(0) == in.size(0) && out.size(1) == in.size(1),
+              "gelu: shapes or dtypes disagree");
+  done(r32_gelu(in.data_ptr(), ldi, out.data_ptr(), ldo, (int)in.size(0), (int)in.size(1), f, stream()), "gelu");
+}
+
+const float* opt_f32(const c10::optional<Tensor>& t, int64_t n, const char* name) {
+  if (!t.has_value()) return nullptr;
+  want(*t, torch::kFloat32, name);
+  TORCH_CHECK(t->numel() == n, name, ": wrong size");
+  return t->data_ptr<float>();
+}
+
+// src rows [q (H D) | k (G D) | v (G Dv)] (bf16 or fp32); wq / wk fp32 [D] per-head norm weights or absent; freq fp32
+// [rd / 2] (absent when rd == 0), vfreq fp32 [Dv / 2] or absent (values not rotated); q_out fp32 [T, H D]; caches: one
+// layer's views of the paged pool.
+void rot_kv_write(Tensor src, c10::optional<Tensor> wq, c10::optional<Tensor> wk, c10::optional<Tensor> freq, double mult,
+                  int64_t rd, c10::optional<Tensor> vfreq, Tensor positions, Tensor slots, Tensor q_out, Tensor k_cache,
+                  Tensor v_cache, int64_t H, int64_t G, double eps, double scale) {
+  const int fi = act_f32(src, "rot_kv_write src"), fc = act_f32(k_cache, "rot_kv_write k_cache");
+  const int lds = row_stride(src, "rot_kv_write src");
+  const int T = (int)src.size(0);
+  want(positions, torch::kInt32, "rot_kv_write positions");
+  want(slots, torch::kInt32, "rot_kv_write slots");
+  want(q_out, torch::kFloat32, "rot_kv_write q_out");
+  TORCH_CHECK(v_cache.is_cuda() && v_cache.scalar_type() == k_cache.scalar_type() && (fi || !fc),
+              "rot_kv_write: caches of one dtype, bf16 rows only into a bf16 cache");
+  int NB, BS, nk, nv;
+  cache_layout(k_cache, v_cache, NB, BS, nk, nv, "rot_kv_write");
+  TORCH_CHECK(H > 0 && G > 0 && H % G == 0 && nk % G == 0 && nv % G == 0, "rot_kv_write: head counts");
+  const int D = nk / (int)G, Dv = nv / (int)G;
+  TORCH_CHECK(src.size(1) == H * D + nk + nv && positions.numel() == T && slots.numel() == T &&
+                  q_out.numel() == (int64_t)T * H * D && rd >= 0 && rd <= D && rd % 2 == 0 && (rd == 0 || freq.has_value()) &&
+                  (!vfreq.has_value() || Dv % 2 == 0), "rot_kv_write: shapes disagree");
+  done(r32_rot_kv_write(src.data_ptr(), lds, opt_f32(wq, D, "rot_kv_write wq"), opt_f32(wk, D, "rot_kv_write wk"),
+                        opt_f32(freq, rd / 2, "rot_kv_write freq"), (float)mult, (int)rd, opt_f32(vfreq, Dv / 2, "rot_kv_write vfreq"),
+                        positions.data_ptr<int>(), slots.data_ptr<int>(), q_out.data_ptr<float>(), k_cache.data_ptr(),
+                        v_cache.data_ptr(), (long long)k_cache.stride(0), (long long)v_cache.stride(0), BS, T, (int)H, (int)G, D,
+                        Dv, (float)eps, (float)scale, fi | (fc << 1), stream()), "rot_kv_write");
+}
+
+// o, out [T, H Dv] row-dense views of one dtype (not the same memory); g [T, >= H] gate logits or absent
+void head_gate_unrotate(Tensor o, c10::optional<Tensor> g, c10::optional<Tensor> vfreq, Tensor positions, Tensor out,
+                        int64_t H, double scale) {
+  const int f = act_f32(o, "head_gate_unrotate o");
+  const int ldi = row_stride(o, "head_gate_unrotate o"), ldo = row_stride(out, "head_gate_unrotate out");
+  want(positions, torch::kInt32, "head_gate_unrotate positions");
+  const int T = (int)o.size(0);
+  TORCH_CHECK(out.is_cuda() && out.scalar_type() == o.scalar_type() && out.size(0) == T && out.size(1) == o.size(1) && H > 0 &&
+                  o.size(1) % H == 0 && positions.numel() == T && out.data_ptr() != o.data_ptr(), "head_gate_unrotate: shapes");
+  const int Dv = (int)(o.size(1) / H);
+  const void* gp = nullptr;
+  int ldg = 0;
+  if (g.has_value()) {
+    TORCH_CHECK(g->is_cuda() && g->scalar_type() == o.scalar_type() && g->size(0) == T && g->size(1) == H, "head_gate_unrotate: g");
+    ldg = row_stride(*g, "head_gate_unrotate g");
+    gp = g->data_ptr();
+  }
+  done(r32_head_gate_unrotate(o.data_ptr(), ldi, gp, ldg, opt_f32(vfreq, Dv / 2, "head_gate_unrotate vfreq"),
+                              positions.data_ptr<int>(), out.data_ptr(), ldo, T, (int)H, Dv, (float)scale, f, stream()),
+       "head_gate_unrotate");
+}
+
+// x fp32 [T, d] += y (absent: x stays); out = x / rms(x) * w (bf16 or fp32 rows)
+void add_rmsnorm(Tensor x, c10::optional<Tensor> y, Tensor w, Tensor out, double eps) {
+  want(x, torch::kFloat32, "add_rmsnorm x");
+  want(w, torch::kFloat32, "add_rmsnorm w");
+  const int fo = act_f32(out, "add_rmsnorm out");
+  const int ldo = row_stride(out, "add_rmsnorm out");
+  TORCH_CHECK(x.dim() == 2 && out.size(0) == x.size(0) && out.size(1) == x.size(1) && w.numel() == x.size(1), "add_rmsnorm: shapes");
+  const void* yp = nullptr;
+  int ldy = 0, fy = 0;
+  if (y.has_value()) {
+    fy = act_f32(*y, "add_rmsnorm y");
+    ldy = row_stride(*y, "add_rmsnorm y");
+    TORCH_CHECK(y->size(0) == x.size(0) && y->size(1) == x.size(1), "add_rmsnorm: y");
+    yp = y->data_ptr();
+  }
+  done(r32_add_rmsnorm(x.data_ptr<float>(), yp, ldy, w.data_ptr<float>(), out.data_ptr(), ldo, (int)x.size(0), (int)x.size(1),
+                       (float)eps, fy | (fo << 1), stream()), "add_rmsnorm");
+}
+
+int64_t chan_rule_max_dim() { return r32_chan_rule_max_dim(); }
+
+// src [T, 2 G D + H Dv] rows [q | k | v] (bf16 or fp32); qkv fp32 of the same shape (src itself when that is fp32);
+// z [T, H D] decay logits, zb fp32 [H D] or absent; A_log fp32 [H] (delta-rule decays) or absent (sigmoid^(1/tau));
+// b [T, >= H] beta logits or absent; state fp32 [slots, H, D, Dv] view; out fp32 [T, H Dv].
+void chan_rule(Tensor src, Tensor qkv, Tensor z, c10::optional<Tensor> zb, c10::optional<Tensor> A_log, double inv_tau,
+               c10::optional<Tensor> b, Tensor state, Tensor cu, Tensor item_slot, Tensor positions, Tensor out, int64_t H,
+               int64_t G, bool unit, bool delta) {
+  const int fs = act_f32(src, "chan_rule src"), fz = act_f32(z, "chan_rule z");
+  const int lds = row_stride(src, "chan_rule src"), ldz = row_stride(z, "chan_rule z");
+  want_dev(qkv, torch::kFloat32, "chan_rule qkv");
+  const int ldq = row_stride(qkv, "chan_rule qkv");
+  want_dev(state, torch::kFloat32, "chan_rule state");
+  want(cu, torch::kInt32, "chan_rule cu");
+  want(item_slot, torch::kInt32, "chan_rule item_slot");
+  want(positions, torch::kInt32, "chan_rule positions");
+  want_dev(out, torch::kFloat32, "chan_rule out");
+  const int ldo = row_stride(out, "chan_rule out");
+  TORCH_CHECK(state.dim() == 4 && state.size(1) == H && state.stride(3) == 1 && state.stride(2) == state.size(3) &&
+                  state.stride(1) == state.size(2) * state.size(3), "chan_rule: state [slots, H, D, Dv]");
+  const int D = (int)state.size(2), Dv = (int)state.size(3), T = (int)src.size(0);
+  TORCH_CHECK(G > 0 && H % G == 0 && src.size(1) == 2 * G * D + H * Dv && qkv.size(0) == T && qkv.size(1) == src.size(1) &&
+                  out.size(0) == T && out.size(1) == H * Dv && z.size(0) == T && z.size(1) == H * D && positions.numel() == T &&
+                  cu.numel() == item_slot.numel() + 1 && D <= r32_chan_rule_max_dim() &&
+                  (fs || src.data_ptr() != qkv.data_ptr()), "chan_rule: shapes disagree");
+  const void* bp = nullptr;
+  int ldb = 0, fb = 0;
+  if (b.has_value()) {
+    fb = act_f32(*b, "chan_rule b");
+    ldb = row_stride(*b, "chan_rule b");
+    TORCH_CHECK(b->size(0) == T && b->size(1) == H, "chan_rule: b [T, H]");
+    bp = b->data_ptr();
+  }
+  Tensor dec = torch::empty({T, H * D}, qkv.options().dtype(torch::kFloat32));
+  Tensor bq = torch::empty({T, H + G}, dec.options());
+  done(r32_chan_rule(src.data_ptr(), lds, fs, qkv.data_ptr<float>(), ldq, z.data_ptr(), ldz, fz,
+                     opt_f32(zb, H * D, "chan_rule zb"), opt_f32(A_log, H, "chan_rule A_log"), (float)inv_tau, bp, ldb, fb,
+                     dec.data_ptr<float>(), bq.data_ptr<float>(), state.data_ptr<float>(), (long long)state.stride(0),
+                     cu.data_ptr<int>(), item_slot.data_ptr<int>(), positions.data_ptr<int>(), out.data_ptr<float>(), ldo, T,
+                     (int)item_slot.numel(), (int)H, (int)G, D, Dv, unit ? 1 : 0, delta ? 1 : 0, stream()), "chan_rule");
+}
+
 }  // namespace
 
 PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
@@ -802,4 +941,10 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
   m.def("retention", &retention);
   m.def("retention_max_dim", &retention_max_dim);
   m.def("glu", &glu);
+  m.def("gelu", &gelu);
+  m.def("rot_kv_write", &rot_kv_write);
+  m.def("head_gate_unrotate", &head_gate_unrotate);
+  m.def("add_rmsnorm", &add_rmsnorm);
+  m.def("chan_rule", &chan_rule);
+  m.def("chan_rule_max_dim", &chan_rule_max_dim);
 }

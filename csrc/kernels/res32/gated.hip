@@ -1,6 +1,6 @@
 // Layer plumbing of fp32-residual designs with gated, post-normalised sublayers (gfx950, wave64).
 //
-//   embed_rows           x[t] = table[token[t]] as fp32
+//   embed_rows           x[t] = table[token[t]] * scale as fp32
 //   head_norm_kv_write   from fused projection rows: q and k divided by their root mean square PER HEAD (no weight);
 //                        q times scale * (1 + coef ln(floor((p + 1) / every) + 1)) into an fp32 buffer; normalised k
 //                        into the paged K cache; the values (a projection of their own, or the keys as projected,
@@ -18,12 +18,12 @@ namespace {
 
 template <typename AT>
 __global__ void embed_rows_kernel(const AT* __restrict__ table, const int* __restrict__ tokens, float* __restrict__ out,
-                                  int d, int vocab) {
+                                  int d, int vocab, float scale) {
   const int t = blockIdx.x;
   int tok = tokens[t];
   tok = tok < 0 ? 0 : (tok >= vocab ? vocab - 1 : tok);
   const AT* row = table + (size_t)tok * d;
-  for (int i = threadIdx.x; i < d; i += blockDim.x) out[(size_t)t * d + i] = Elem<AT>::ld(row + i);
+  for (int i = threadIdx.x; i < d; i += blockDim.x) out[(size_t)t * d + i] = Elem<AT>::ld(row + i) * scale;
 }
 
 // proj row t: q at column 0 (H*D), k at k_off (G*D), values at v_off (G*Dv; v_off == k_off: the keys as projected).
@@ -290,11 +290,11 @@ int blocks_for(long long total) { return (int)((total + 255) / 256 < 65536 ? (to
 
 using namespace lwc;
 
-extern "C" int r32_embed_rows(const void* table, const int* tokens, float* out, int T, int d, int vocab, int f32,
-                              hipStream_t s) {
+extern "C" int r32_embed_rows(const void* table, const int* tokens, float* out, int T, int d, int vocab, float scale,
+                              int f32, hipStream_t s) {
   if (T <= 0) return 0;
-  if (f32) embed_rows_kernel<float><<<T, 256, 0, s>>>((const float*)table, tokens, out, d, vocab);
-  else embed_rows_kernel<bf16_t><<<T, 256, 0, s>>>((const bf16_t*)table, tokens, out, d, vocab);
+  if (f32) embed_rows_kernel<float><<<T, 256, 0, s>>>((const float*)table, tokens, out, d, vocab, scale);
+  else embed_rows_kernel<bf16_t><<<T, 256, 0, s>>>((const bf16_t*)table, tokens, out, d, vocab, scale);
   LWC_CHECK_LAUNCH();
   return 0;
 }

@@ -3,6 +3,8 @@
 //   mode 0   y = silu(g) * u
 //   mode 1   g' = min(g, L), u' = clamp(u, -L, L);  y = g' * sigmoid(alpha g') * (u' + 1)      (clamped gate unit)
 // in: rows [gate (n) | up (n)] with leading dimension ldi; out: rows of n (leading dimension ldo).
+//
+//   gelu     y = z / 2 (1 + erf(z / sqrt(2))) over rows of n (an ungated feed-forward's activation)
 #include "elem.h"
 
 namespace lwc {
@@ -37,6 +39,27 @@ __global__ void glu_vec_kernel(const AT* __restrict__ in, int ldi, AT* __restric
     const float4v g = Vec4<AT>::ld(r + c), u = Vec4<AT>::ld(r + 4 * n4 + c);
     Vec4<AT>::st(out + t * ldo + c, float4v{glu_f<MODE>(g[0], u[0], alpha, limit), glu_f<MODE>(g[1], u[1], alpha, limit),
                                             glu_f<MODE>(g[2], u[2], alpha, limit), glu_f<MODE>(g[3], u[3], alpha, limit)});
+  }
+}
+
+LWC_DEVICE float gelu_erf_f(float z) { return 0.5f * z * (1.0f + erff(z * 0.7071067811865476f)); }
+
+template <typename AT>
+__global__ void gelu_kernel(const AT* __restrict__ in, int ldi, AT* __restrict__ out, int ldo, int n, long long total) {
+  for (long long e = (long long)blockIdx.x * blockDim.x + threadIdx.x; e < total; e += (long long)gridDim.x * blockDim.x) {
+    const long long t = e / n;
+    const int c = (int)(e - t * n);
+    Elem<AT>::st(out + t * ldo + c, gelu_erf_f(Elem<AT>::ld(in + t * ldi + c)));
+  }
+}
+
+template <typename AT>
+__global__ void gelu_vec_kernel(const AT* __restrict__ in, int ldi, AT* __restrict__ out, int ldo, int n4, long long total4) {
+  for (long long e = (long long)blockIdx.x * blockDim.x + threadIdx.x; e < total4; e += (long long)gridDim.x * blockDim.x) {
+    const long long t = e / n4;
+    const int c = 4 * (int)(e - t * n4);
+    const float4v z = Vec4<AT>::ld(in + t * ldi + c);
+    Vec4<AT>::st(out + t * ldo + c, float4v{gelu_erf_f(z[0]), gelu_erf_f(z[1]), gelu_erf_f(z[2]), gelu_erf_f(z[3])});
   }
 }
 
@@ -77,6 +100,19 @@ extern "C" int r32_glu(const void* in, int ldi, void* out, int ldo, int T, int n
     }
   }
 #undef LWC_GLU
+  LWC_CHECK_LAUNCH();
+  return 0;
+}
+
+extern "C" int r32_gelu(const void* in, int ldi, void* out, int ldo, int T, int n, int f32, hipStream_t s) {
+  const long long total = (long long)T * n;
+  if (total <= 0) return 0;
+  const int ab = f32 ? 16 : 8;
+  const bool vec = n % 4 == 0 && ldi % 4 == 0 && ldo % 4 == 0 && aligned_to(in, ab) && aligned_to(out, ab);
+  if (vec && f32) gelu_vec_kernel<float><<<glu_grid(total / 4), 256, 0, s>>>((const float*)in, ldi, (float*)out, ldo, n / 4, total / 4);
+  else if (vec) gelu_vec_kernel<bf16_t><<<glu_grid(total / 4), 256, 0, s>>>((const bf16_t*)in, ldi, (bf16_t*)out, ldo, n / 4, total / 4);
+  else if (f32) gelu_kernel<float><<<glu_grid(total), 256, 0, s>>>((const float*)in, ldi, (float*)out, ldo, n, total);
+  else gelu_kernel<bf16_t><<<glu_grid(total), 256, 0, s>>>((const bf16_t*)in, ldi, (bf16_t*)out, ldo, n, total);
   LWC_CHECK_LAUNCH();
   return 0;
 }

@@ -6,7 +6,7 @@
 //
 //   conv_hist         causal convolution over time per channel, y_t = sum_s w[c][taps-1-s] x_(t-s), s < taps; the
 //                     inputs before the item's first row come from the slot's history (the last taps-1 inputs).
-//                     MODE 0: out = x + y (and optionally a cast copy of x); MODE 1: out = silu(y)
+//                     MODE 0: out = x + y (and optionally a cast copy of x); MODE 1: out = silu(y); MODE 2: out = y
 //   conv_hist_update  the slot's history after the step: the last taps-1 inputs of old history ++ this step's rows
 //   delta_rule        gated delta rule, one wave per (item, head, 16 value columns), a quarter state column per lane:
 //                       S <- g S;  u = beta (v - S^T k);  S <- S + k u^T;  o = S^T q
@@ -51,7 +51,7 @@ __global__ void conv_hist_kernel(const IT* __restrict__ x, int ldx, const float*
     Elem<OT>::st(out + (size_t)t * ldo + c, cur + acc);
     if (out2) Elem<OT>::st(out2 + (size_t)t * ldo2 + c, cur);
   } else {
-    Elem<OT>::st(out + (size_t)t * ldo + c, silu_f(acc));
+    Elem<OT>::st(out + (size_t)t * ldo + c, MODE == 1 ? silu_f(acc) : acc);
   }
 }
 
@@ -90,7 +90,7 @@ __global__ void conv_hist_vec_kernel(const IT* __restrict__ x, int ldx, const fl
     Vec4<OT>::st(out + (size_t)t * ldo + c, cur + acc);
     if (out2) Vec4<OT>::st(out2 + (size_t)t * ldo2 + c, cur);
   } else {
-    Vec4<OT>::st(out + (size_t)t * ldo + c, float4v{silu_f(acc[0]), silu_f(acc[1]), silu_f(acc[2]), silu_f(acc[3])});
+    Vec4<OT>::st(out + (size_t)t * ldo + c, MODE == 1 ? float4v{silu_f(acc[0]), silu_f(acc[1]), silu_f(acc[2]), silu_f(acc[3])} : acc);
   }
 }
 
@@ -134,7 +134,7 @@ __global__ void conv_hist_tile_kernel(const IT* __restrict__ x, int ldx, const f
       Vec4<OT>::st(out + (size_t)t * ldo + c, cur + acc);
       if (out2) Vec4<OT>::st(out2 + (size_t)t * ldo2 + c, cur);
     } else {
-      Vec4<OT>::st(out + (size_t)t * ldo + c, float4v{silu_f(acc[0]), silu_f(acc[1]), silu_f(acc[2]), silu_f(acc[3])});
+      Vec4<OT>::st(out + (size_t)t * ldo + c, MODE == 1 ? float4v{silu_f(acc[0]), silu_f(acc[1]), silu_f(acc[2]), silu_f(acc[3])} : acc);
     }
 #pragma unroll
     for (int s = 6; s >= 1; --s) prev[s] = prev[s - 1];
@@ -437,7 +437,7 @@ extern "C" int r32_conv_hist(const void* x, int ldx, const float* w, int ws_c, i
     } else {
       return -1;
     }
-  } else {
+  } else if (mode == 1) {
     if (io == 3) {
       LWC_CONV(float, float, 1);
     } else if (io == 2) {
@@ -447,6 +447,18 @@ extern "C" int r32_conv_hist(const void* x, int ldx, const float* w, int ws_c, i
     } else {
       return -1;
     }
+  } else if (mode == 2) {
+    if (io == 3) {
+      LWC_CONV(float, float, 2);
+    } else if (io == 2) {
+      LWC_CONV(bf16_t, float, 2);
+    } else if (io == 0) {
+      LWC_CONV(bf16_t, bf16_t, 2);
+    } else {
+      return -1;
+    }
+  } else {
+    return -1;
   }
 #undef LWC_CONV
   LWC_CHECK_LAUNCH();

@@ -71,7 +71,7 @@ window_attn_kernel(const float* __restrict__ q, const CT* __restrict__ k_cache, 
                    long long kb_stride, long long vb_stride, int block_size, const int* __restrict__ positions,
                    const int* __restrict__ cu_q, int n_items, const int* __restrict__ block_tables, int bt_width,
                    const float* __restrict__ r1, const float* __restrict__ r2, const float* __restrict__ sink, int window,
-                   CT* __restrict__ out, int ldo, int H, int G, int D, int Dv) {
+                   int chunk, CT* __restrict__ out, int ldo, int H, int G, int D, int Dv) {
   extern __shared__ float q_s[];  // [D]
   __shared__ float p_s[64];
   __shared__ long long vo_s[64];
@@ -101,7 +101,7 @@ window_attn_kernel(const float* __restrict__ q, const CT* __restrict__ k_cache, 
 #pragma unroll
   for (int ns = 0; ns < kMaxSlots; ++ns) o[ns] = 0.f;
   float m = -INFINITY, l = 0.f;
-  const int j_lo = max(0, i - window + 1);
+  const int j_lo = max(max(0, i - window + 1), chunk > 0 ? i - i % chunk : 0);  // the window's and the chunk's first key
   for (int j0 = j_lo; j0 <= i; j0 += 64) {
     const int j = j0 + lane;
     const bool valid = j <= i;
@@ -162,7 +162,7 @@ using namespace lwc;
 extern "C" int r32_window_attn(const float* q, const void* k_cache, const void* v_cache, long long kb_stride,
                                long long vb_stride, int block_size, const int* positions, const int* cu_q, int n_items,
                                const int* block_tables, int bt_width, const float* r1, const float* r2, const float* sink,
-                               int window, void* out, int ldo, int T, int H, int G, int D, int Dv, int f32, hipStream_t s) {
+                               int window, int chunk, void* out, int ldo, int T, int H, int G, int D, int Dv, int f32, hipStream_t s) {
   if (T <= 0) return 0;
   if (Dv > 64 * kMaxSlots || D > 8192 || H % G != 0) return -1;
   const dim3 grid(T, H);
@@ -170,11 +170,11 @@ extern "C" int r32_window_attn(const float* q, const void* k_cache, const void* 
   if (f32)
     window_attn_kernel<float><<<grid, 64, shm, s>>>(q, (const float*)k_cache, (const float*)v_cache, kb_stride, vb_stride,
                                                     block_size, positions, cu_q, n_items, block_tables, bt_width, r1, r2,
-                                                    sink, window, (float*)out, ldo, H, G, D, Dv);
+                                                    sink, window, chunk, (float*)out, ldo, H, G, D, Dv);
   else
     window_attn_kernel<bf16_t><<<grid, 64, shm, s>>>(q, (const bf16_t*)k_cache, (const bf16_t*)v_cache, kb_stride,
                                                      vb_stride, block_size, positions, cu_q, n_items, block_tables,
-                                                     bt_width, r1, r2, sink, window, (bf16_t*)out, ldo, H, G, D, Dv);
+                                                     bt_width, r1, r2, sink, window, chunk, (bf16_t*)out, ldo, H, G, D, Dv);
   return (int)hipGetLastError();
 }
 
@@ -215,6 +215,7 @@ struct WAttnMfmaParams {
   const float* bias;  // [H, window], or null: no distance bias
   const float* sink;  // [H], or null: exp(sink_h) joins the softmax denominator of head h (no key, no value)
   int window;
+  int chunk;          // > 0: row i sees only keys of its own chunk, j >= i - i % chunk (besides the window)
   bf16_t* out;
   int ldo, H, G;
 };
@@ -240,7 +241,9 @@ __global__ void __launch_bounds__(256) window_attn_mfma_kernel(const WAttnMfmaPa
   const int nrows = min(64, q_end - row0);
   const int k_len = p.k_lens[it];
   const int pos0 = p.positions[row0], pos_last = pos0 + nrows - 1;  // positions ascend by one along the rows
-  const int j_lo = max(0, pos0 - p.window + 1), j_hi = min(pos_last, k_len - 1);
+  // first visible key of the row at position i: the later of its window's and its chunk's start (ascends with i)
+  auto lo_of = [&](int i) { return max(max(0, i - p.window + 1), p.chunk > 0 ? i - i % p.chunk : 0); };
+  const int j_lo = lo_of(pos0), j_hi = min(pos_last, k_len - 1);
   const int tid = threadIdx.x, w = tid >> 6, lane = tid & 63, r16 = lane & 15, g4 = lane >> 4;
   const int* table = p.block_tables + (size_t)it * p.bt_width;
   const int BS = p.block_size, bsh = p.bs_shift;
@@ -265,6 +268,7 @@ __global__ void __launch_bounds__(256) window_attn_mfma_kernel(const WAttnMfmaPa
     }
   }
   const int w_min = pos0 + 16 * w, w_max = min(pos0 + 16 * w + 15, pos_last);  // this wave's positions
+  const int w_lo_min = lo_of(w_min), w_lo_max = lo_of(max(w_max, w_min)), lo_q = lo_of(i_q);  // and their first visible keys
   const bool wave_live = 16 * w < nrows;
 
   float4v O[NV];
@@ -345,7 +349,7 @@ __global__ void __launch_bounds__(256) window_attn_mfma_kernel(const WAttnMfmaPa
     const float* bias_s = bias_s2[cur];
     if (kt < kt_hi) fetch(kt + 1);
     // the tile's keys [32 kt, 32 kt + 31] against this wave's rows: nothing visible -> nothing to compute
-    if (wave_live && kt * 32 <= w_max && kt * 32 + 31 >= w_min - p.window + 1) {
+    if (wave_live && kt * 32 <= w_max && kt * 32 + 31 >= w_lo_min) {
     float4v sacc[2];
 #pragma unroll
     for (int sub = 0; sub < 2; ++sub) {
@@ -358,7 +362,7 @@ __global__ void __launch_bounds__(256) window_attn_mfma_kernel(const WAttnMfmaPa
       }
     }
     // every key of the tile visible to every row of the wave: no masks
-    const bool inner = kt * 32 + 31 <= w_min && kt * 32 >= w_max - p.window + 1 && w_max - w_min == 15;
+    const bool inner = kt * 32 + 31 <= w_min && kt * 32 >= w_lo_max && w_max - w_min == 15;
     float s[8];
     float mx = -1e30f;
     const float* brow = bias_s + (qrow + 31 - 4 * g4);
@@ -373,7 +377,7 @@ __global__ void __launch_bounds__(256) window_attn_mfma_kernel(const WAttnMfmaPa
       for (int e = 0; e < 8; ++e) {
         const int jl = (e >> 2) * 16 + 4 * g4 + (e & 3);
         const int dist = i_q - (kt * 32 + jl);
-        const bool ok = q_valid && dist >= 0 && dist < p.window;
+        const bool ok = q_valid && dist >= 0 && kt * 32 + jl >= lo_q;
         s[e] = ok ? fmaf(sacc[e >> 2][e & 3], kLog2e, -brow[-((e >> 2) * 16 + (e & 3))]) : -1e30f;
         mx = fmaxf(mx, s[e]);
       }
@@ -467,7 +471,7 @@ extern "C" int r32_window_attn_mfma_ok(int D, int Dv) {
 extern "C" int r32_window_attn_mfma(const float* q, const void* k_cache, const void* v_cache, long long kb_stride,
                                     long long vb_stride, int block_size, const int* positions, const int* cu_q,
                                     const int* k_lens, int n_items, int max_q, const int* block_tables, int bt_width,
-                                    const float* bias, const float* sink, int window, void* out, int ldo, int H, int G,
+                                    const float* bias, const float* sink, int window, int chunk, void* out, int ldo, int H, int G,
                                     int D, int Dv, hipStream_t s) {
   if (n_items <= 0 || max_q <= 0) return 0;
   if (!r32_window_attn_mfma_ok(D, Dv) || H % G != 0 || (block_size & (block_size - 1)) != 0) return -1;
@@ -478,7 +482,7 @@ extern "C" int r32_window_attn_mfma(const float* q, const void* k_cache, const v
   for (int b = 0; b < 20; ++b)
     if ((1 << b) == block_size) p.bs_shift = b;
   p.cu_q = cu_q; p.k_lens = k_lens; p.tiles_per_item = (max_q + 63) / 64; p.block_tables = block_tables;
-  p.bt_width = bt_width; p.bias = bias; p.sink = sink; p.window = window; p.out = (bf16_t*)out; p.ldo = ldo; p.H = H; p.G = G;
+  p.bt_width = bt_width; p.bias = bias; p.sink = sink; p.window = window; p.chunk = chunk; p.out = (bf16_t*)out; p.ldo = ldo; p.H = H; p.G = G;
   const dim3 grid(n_items * p.tiles_per_item, H);
   // a workgroup's keys span at most window + 63 positions (from a 32-aligned start: + 31) and never more than the table
   long long span = (long long)window + 63 + 31;

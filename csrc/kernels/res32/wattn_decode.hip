@@ -66,7 +66,7 @@ extern "C" int r32_window_attn_decode_splits(int B, int G, int Hg, int max_keys,
 // the keys any row sees (min(window, longest context)), known on the host.
 extern "C" int r32_window_attn_decode(const float* q, const void* k_cache, const void* v_cache, long long kb_stride,
                                       long long vb_stride, int block_size, const int* positions, const int* block_tables,
-                                      int bt_width, const float* bias, const float* sink, int window, float* part_o,
+                                      int bt_width, const float* bias, const float* sink, int window, int chunk, float* part_o,
                                       float* part_ml, int S, int max_keys, void* out, int ldo, int B, int H, int G, int D,
                                       int Dv, int vk, hipStream_t s) {
   if (B <= 0) return 0;
@@ -77,7 +77,7 @@ extern "C" int r32_window_attn_decode(const float* q, const void* k_cache, const
   p.bs_shift = -1;
   for (int b = 0; b < 20; ++b)
     if ((1 << b) == block_size) p.bs_shift = b;
-  p.bt_width = bt_width; p.bias = bias; p.window = window; p.part_o = part_o; p.part_ml = part_ml; p.H = H; p.G = G;
+  p.bt_width = bt_width; p.bias = bias; p.window = window; p.chunk = chunk; p.part_o = part_o; p.part_ml = part_ml; p.H = H; p.G = G;
   p.S = S;
   // a row's keys start at a multiple of 32 at or below its window's first key: up to max_keys + 31 keys to cover
   p.keys_per_split = (((max_keys + 31 + S - 1) / S) + 31) / 32 * 32;

@@ -30,6 +30,7 @@ struct WAttnDecodeParams {
   int bt_width;
   const float* bias;       // [H, window], or null: no distance bias
   int window;
+  int chunk;               // > 0: the row sees only keys of its own chunk, j >= i - i % chunk (besides the window)
   float* part_o;           // [B, H, S, Dv]
   float* part_ml;          // [B, H, S, 2]
   int H, G, S, keys_per_split;  // keys_per_split: a multiple of 32
@@ -59,7 +60,7 @@ __global__ void __launch_bounds__(64 * NW * NC) window_attn_decode_kernel(const 
   const int nh = min(16, g * Hg + Hg - h0);  // heads of this chunk (<= 0: a wave past the last chunk only helps staging)
   const int r16 = lane & 15, g4 = lane >> 4;
   const int i = p.positions[b];
-  const int j_lo = max(0, i - p.window + 1);
+  const int j_lo = max(max(0, i - p.window + 1), p.chunk > 0 ? i - i % p.chunk : 0);
   const int base = (j_lo / 32) * 32 + split * p.keys_per_split;  // this split's first key (a multiple of 32)
   const int last = min(i, base + p.keys_per_split - 1);
   const int* table = p.block_tables + (size_t)b * p.bt_width;
@@ -175,7 +176,7 @@ __global__ void __launch_bounds__(64 * NW * NC) window_attn_decode_kernel(const 
     for (int e = 0; e < 8; ++e) {
       const int j = t0 + (e >> 2) * 16 + 4 * g4 + (e & 3);
       const int dist = i - j;
-      ok[e] = h_valid && dist >= 0 && dist < p.window && j <= last;
+      ok[e] = h_valid && dist >= 0 && j >= j_lo && j <= last;
       s[e] = ok[e] ? sacc[e >> 2][e & 3] - (bias_h ? bias_h[dist] : 0.f) : -1e30f;
       mx = fmaxf(mx, s[e]);
     }

@@ -561,8 +561,186 @@ class LimatarConfig:
         return n
 
 
+# ------------------------------------------------------------------ Rerozen
+@dataclass(frozen=True)
+class RotaryAttentionSpec:
+    """Causal softmax attention with rotary positions on the first ``rot.dims`` entries of every q / k head (rotate-half
+    pairing), GQA, a sigmoid gate per head on the output.  ``chunk``: positions are cut into chunks of that many from
+    position 0 and a row sees only its own chunk.  Options: biases on q / k / v; a per-head RMS norm of q and k with one
+    weight for all heads (before the rotation); a short causal convolution (``conv`` taps, 0 = none) behind the three
+    projections; values rotated by their own position over all ``vdim`` entries (plain frequencies of ``rot.base``) and
+    the head's output turned back by the query's position; ``sink``: one added to the softmax's denominator."""
+    heads: int
+    kv_heads: int
+    dim: int
+    vdim: int
+    scale: float
+    chunk: int
+    rot: RotarySpec
+    bias: bool = False
+    qk_norm: bool = False
+    conv: int = 0
+    rotate_values: bool = False
+    sink: bool = False
+
+    @property
+    def nq(self) -> int:
+        return self.heads * self.dim
+
+    @property
+    def nk(self) -> int:
+        return self.kv_heads * self.dim
+
+    @property
+    def nv(self) -> int:
+        return self.kv_heads * self.vdim
+
+
+@dataclass(frozen=True)
+class ChannelDecaySpec:
+    """A linear-attention mixer whose state rows decay per head AND key channel; the decay logits come through a low-rank
+    pair of projections (``a_rank``; 0: read from the checkpoint's tensor shapes).
+    ``kind`` "gla": S <- diag(alpha) S + k v^T with alpha = sigmoid(z)^(1/tau), q times dim^-1/2, silu gate, ``kv_heads``
+    = ``heads``.  ``kind`` "delta": the gated delta rule with unit q / k behind a short convolution (``conv`` taps) + silu,
+    q / k over ``kv_heads`` heads, decays exp(-exp(A_log) softplus(z + dt_bias)), a low-rank sigmoid gate (``g_rank``)."""
+    kind: str
+    heads: int
+    kv_heads: int
+    dim: int
+    vdim: int
+    tau: float = 1.0
+    conv: int = 0
+    a_rank: int = 0
+    g_rank: int = 0
+
+    @property
+    def nq(self) -> int:
+        return self.kv_heads * self.dim
+
+    @property
+    def nv(self) -> int:
+        return self.heads * self.vdim
+
+    @property
+    def nd(self) -> int:
+        return self.heads * self.dim
+
+
+@dataclass(frozen=True)
+class RerozenLayerSpec:
+    type: str                       # "parallel" (attention beside gated linear attention) | "parallel_2" (... delta rule)
+    left: RotaryAttentionSpec
+    right: ChannelDecaySpec
+    left_scale: float
+    right_scale: float
+    ff: int                         # 0: no feed-forward in this layer
+
+    @property
+    def mixer(self) -> RotaryAttentionSpec:
+        return self.left
+
+
+@dataclass(frozen=True)
+class RerozenConfig:
+    """Rerozen: a pre-norm fp32 residual stream; every sublayer reads h + causal_conv(h) of its normed input; a mixer is
+    TWO mixers side by side on the same input, a chunked rotary attention and a channel-decay linear attention, their
+    results added with fixed scales; ungated gelu feed-forwards; scaled embedding and logits."""
+    name: str
+    vocab_size: int
+    hidden: int
+    layer_specs: Tuple[RerozenLayerSpec, ...]
+    norm_eps: float
+    canon_taps: int
+    embed_scale: float
+    logit_scale: float
+    bos_token_id: int = 1
+    eos_token_id: int = 2
+
+    architecture = "Rerozen"
+    num_experts = 0   # the engine's expert-parallel planning does not apply
+
+    @property
+    def layers(self) -> int:
+        return len(self.layer_specs)
+
+    @property
+    def heads(self) -> int:
+        return max(L.left.heads for L in self.layer_specs)
+
+    @property
+    def kv_heads(self) -> int:
+        return max(L.left.kv_heads for L in self.layer_specs)
+
+    @property
+    def head_dim(self) -> int:
+        return max(L.left.dim for L in self.layer_specs)
+
+    @classmethod
+    def from_dict(cls, c: dict, name: str = "rerozen") -> "RerozenConfig":
+        specs = []
+        for L in c["layers"]:
+            if L["type"] not in ("parallel", "parallel_2"):
+                raise ValueError(f"Rerozen: unknown mixer type {L['type']!r}")
+            two = L["type"] == "parallel_2"
+            m = L["mixer"]
+            a, b = m["left"], m["right"]
+            rot = RotarySpec.from_dict(a["rot"])
+            left = RotaryAttentionSpec(heads=int(a["heads"]), kv_heads=int(a["kv_heads"]), dim=int(a["dim"]), vdim=int(a["vdim"]),
+                                       scale=float(a["scale"]), chunk=int(a["mask"]["size"]), rot=rot, bias=not two,
+                                       qk_norm=not two, conv=int(a["conv"]) if two else 0, rotate_values=two, sink=two)
+            if left.heads % left.kv_heads:
+                raise ValueError("Rerozen: heads must be a multiple of kv_heads")
+            if rot.dims % 2 or rot.dims > left.dim or left.chunk < 1 or (two and (left.vdim % 2 or left.conv < 1)):
+                raise ValueError("Rerozen: rot.dims even and at most dim, mask.size >= 1, rotated values of even size")
+            if two:
+                right = ChannelDecaySpec("delta", heads=int(b["heads"]), kv_heads=int(b["kv_heads"]), dim=int(b["dim"]),
+                                         vdim=int(b["vdim"]), conv=int(b["conv"]), a_rank=int(b.get("a_rank", 0)),
+                                         g_rank=int(b.get("g_rank", 0)))
+                if right.conv < 1:
+                    raise ValueError("Rerozen: conv taps must be at least 1")
+            else:
+                right = ChannelDecaySpec("gla", heads=int(b["heads"]), kv_heads=int(b["heads"]), dim=int(b["dim"]),
+                                         vdim=int(b["vdim"]), tau=float(b["tau"]), a_rank=int(b.get("a_rank", 0)))
+            if right.heads % right.kv_heads:
+                raise ValueError("Rerozen: heads must be a multiple of kv_heads")
+            mlp = L.get("mlp")
+            if mlp is not None and mlp.get("kind") != "dense":
+                raise ValueError(f"Rerozen: unknown feed-forward kind {mlp.get('kind')!r}")
+            specs.append(RerozenLayerSpec(L["type"], left, right, float(m["left_scale"]), float(m["right_scale"]),
+                                          0 if mlp is None else int(mlp["ff"])))
+        return cls(name=name, vocab_size=int(c["vocab"]), hidden=int(c["width"]), layer_specs=tuple(specs),
+                   norm_eps=float(c["norm"]["eps"]), canon_taps=int(c["canon"]["taps"]),
+                   embed_scale=float(c["embedding"]["scale"]), logit_scale=float(c["logit_scale"]))
+
+    def with_ranks(self, shapes: dict) -> "RerozenConfig":
+        """The config with every low-rank width that it leaves open taken from a checkpoint's tensor shapes."""
+        specs = []
+        for i, L in enumerate(self.layer_specs):
+            r, p = L.right, f"l{i}.mix.right."
+            ar = r.a_rank or int(shapes[p + "a1"][0])
+            gr = r.g_rank or (int(shapes[p + "g1"][0]) if r.kind == "delta" else 0)
+            specs.append(replace(L, right=replace(r, a_rank=ar, g_rank=gr)))
+        return replace(self, layer_specs=tuple(specs))
+
+    def params(self) -> int:
+        d = self.hidden
+        n = 2 * self.vocab_size * d + d
+        for L in self.layer_specs:
+            a, r = L.left, L.right
+            n += d + d * self.canon_taps + d * (a.nq + a.nk + a.nv + a.heads) + d * a.heads * a.vdim
+            n += (a.nq + a.nk + a.nv) * (a.conv + (1 if a.bias else 0)) + (2 * a.dim if a.qk_norm else 0)
+            n += d * (2 * r.nq + r.nv) + d * r.nv + r.vdim + d * r.a_rank + r.a_rank * r.nd + r.nd
+            if r.kind == "delta":
+                n += (2 * r.nq + r.nv) * r.conv + d * r.heads + r.heads + d * r.g_rank + r.g_rank * r.nv
+            else:
+                n += d * r.nv
+            if L.ff:
+                n += d + d * self.canon_taps + 2 * d * L.ff
+        return n
+
+
 # config.json "architecture" -> config class of the layer-list decoders
-ARCHITECTURES = {"Madipel": MadipelConfig, "Merudra": MerudraConfig, "Limatar": LimatarConfig}
+ARCHITECTURES = {"Madipel": MadipelConfig, "Merudra": MerudraConfig, "Limatar": LimatarConfig, "Rerozen": RerozenConfig}
 
 
 def load_model_config(model_dir) -> object:

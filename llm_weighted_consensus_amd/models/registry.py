@@ -12,7 +12,8 @@ from typing import Optional
 
 import torch
 
-from .config import DECODERS, LimatarConfig, MadipelConfig, MerudraConfig, decoder_config, load_model_config
+from .config import (DECODERS, LimatarConfig, MadipelConfig, MerudraConfig, RerozenConfig, decoder_config,
+                     load_model_config)
 
 DTYPES = {"bfloat16": torch.bfloat16, "bf16": torch.bfloat16, "float32": torch.float32, "fp32": torch.float32}
 
@@ -37,6 +38,10 @@ def model_class(cfg):
         from .limatar import LimatarModel
 
         return LimatarModel
+    if isinstance(cfg, RerozenConfig):
+        from .rerozen import RerozenModel
+
+        return RerozenModel
     if getattr(cfg, "num_experts", 0):
         from .mixtral import MixtralModel
 
@@ -52,7 +57,7 @@ def load_model(model_dir: str, device="cuda", dtype=torch.bfloat16, max_position
     instead of the folder's."""
     cfg = load_model_config(model_dir)
     cls = model_class(cfg)
-    if dtype != torch.bfloat16 and not isinstance(cfg, (MadipelConfig, MerudraConfig, LimatarConfig)):
+    if dtype != torch.bfloat16 and not isinstance(cfg, (MadipelConfig, MerudraConfig, LimatarConfig, RerozenConfig)):
         raise ValueError(f"{cfg.name}: this decoder runs in bfloat16 only")
     path = None if random_seed is not None else str(Path(model_dir))
     return cls(cfg, device=device, dtype=dtype, seed=random_seed or 0, weights_path=path, max_position=max_position)

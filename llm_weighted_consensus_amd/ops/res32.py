@@ -105,7 +105,7 @@ def window_attn(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, p
                 block_tables: torch.Tensor, r1: torch.Tensor, r2: torch.Tensor, window: int, out: torch.Tensor,
                 H: int, G: int, cu_q: Optional[torch.Tensor] = None, k_lens: Optional[torch.Tensor] = None,
                 max_q: int = 0, bias: Optional[torch.Tensor] = None, cores: Optional[bool] = None,
-                sink: Optional[torch.Tensor] = None, values_in_keys: bool = False) -> torch.Tensor:
+                sink: Optional[torch.Tensor] = None, values_in_keys: bool = False, chunk: int = 0) -> torch.Tensor:
     """Sliding-window attention over the paged cache with the bias -r1_h ln(1 + r2_h (i - j)); ``q`` fp32
     [T, H*D] pre-scaled; row t reads table row t (``cu_q`` None) or the item whose ``cu_q`` range holds t.
     Over a bf16 cache whose sizes the matrix-core kernels are built for, prompt portions run on the portion kernel
@@ -115,21 +115,24 @@ def window_attn(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, p
     ``sink`` (fp32 [H]): exp(sink_h) joins head h's softmax denominator; it has no key and no value.
     ``values_in_keys``: the caller guarantees that every token's value row repeats the first Dv entries of its key row
     (a cached latent that is key and value at once); the decode kernel for one wide row (576 / 512) then takes its
-    values from the key rows."""
+    values from the key rows.
+    ``chunk`` > 0: positions are cut into chunks of that many, counted from position 0, and a row sees only keys of its
+    own chunk (j >= i - i % chunk), besides the window."""
     K = kernels()
     bs = k_cache.shape[1]
     D, Dv = k_cache.shape[2] // G, v_cache.shape[2] // G
     cores = (bias is not None or bool(cores)) and k_cache.dtype == torch.bfloat16 and bs & (bs - 1) == 0
     if cores and cu_q is None and positions.numel() > 0 and K.window_attn_decode_ok(D, Dv, bool(values_in_keys)):
-        max_keys = min(int(window), block_tables.shape[1] * k_cache.shape[1])
+        max_keys = min(int(window), block_tables.shape[1] * k_cache.shape[1], int(chunk) if chunk > 0 else 1 << 30)
         K.window_attn_decode(q, k_cache, v_cache, positions, block_tables, bias, int(window), max_keys, out, int(H), int(G),
-                             sink, bool(values_in_keys))
+                             sink, bool(values_in_keys), int(chunk))
         return out
     if cores and cu_q is not None and k_lens is not None and max_q > 0 and K.window_attn_mfma_ok(D, Dv):
         K.window_attn_mfma(q, k_cache, v_cache, positions, cu_q, k_lens, int(max_q), block_tables, bias, int(window), out,
-                           int(H), int(G), sink)
+                           int(H), int(G), sink, int(chunk))
         return out
-    K.window_attn(q, k_cache, v_cache, positions, cu_q, block_tables, r1, r2, int(window), out, int(H), int(G), sink)
+    K.window_attn(q, k_cache, v_cache, positions, cu_q, block_tables, r1, r2, int(window), out, int(H), int(G), sink,
+                  int(chunk))
     return out
 
 
@@ -160,7 +163,7 @@ def conv_hist(x: torch.Tensor, w: torch.Tensor, hist: torch.Tensor, items: StepI
               mode: int = 0, out2: Optional[torch.Tensor] = None, update: bool = True) -> torch.Tensor:
     """Causal convolution over time per channel with the inputs before a portion's first row taken from the
     sequence's slot of ``hist`` (fp32 [slots, taps - 1, C]); ``w`` fp32 [C, taps], last column = the current
-    row's.  ``mode`` 0: out = x + conv(x) (``out2``: a copy of x in out's dtype); 1: out = silu(conv(x)).
+    row's.  ``mode`` 0: out = x + conv(x) (``out2``: a copy of x in out's dtype); 1: out = silu(conv(x)); 2: out = conv(x).
     With ``update`` the slot then holds the last taps - 1 inputs after this step."""
     K = kernels()
     fused = bool(update and items.single)  # a decode step: one kernel computes and moves the history on
@@ -191,11 +194,12 @@ def head_norm_gate(o: torch.Tensor, out: torch.Tensor, H: int, eps: float, w: Op
     return out
 
 
-def embed_rows(table: torch.Tensor, tokens: torch.Tensor, out: Optional[torch.Tensor] = None) -> torch.Tensor:
-    """x[t] = table[tokens[t]] as fp32."""
+def embed_rows(table: torch.Tensor, tokens: torch.Tensor, out: Optional[torch.Tensor] = None,
+               scale: float = 1.0) -> torch.Tensor:
+    """x[t] = table[tokens[t]] * scale as fp32."""
     if out is None:
         out = torch.empty(tokens.numel(), table.shape[1], dtype=torch.float32, device=table.device)
-    kernels().embed_rows(table, tokens, out)
+    kernels().embed_rows(table, tokens, out, float(scale))
     return out
 
 
@@ -349,4 +353,67 @@ def glu(gu: torch.Tensor, out: Optional[torch.Tensor] = None, mode: str = "silu"
     if out is None:
         out = torch.empty(gu.shape[0], gu.shape[1] // 2, dtype=gu.dtype, device=gu.device)
     kernels().glu(gu, out, 0 if mode == "silu" else 1, float(alpha), float(limit))
+    return out
+
+
+# ------------------------------------------------------------------ rotary attention layers, channel-wise decays
+def gelu(z: torch.Tensor, out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """z / 2 (1 + erf(z / sqrt 2)); ``z`` and ``out`` may be column slices of row-dense buffers."""
+    if out is None:
+        out = torch.empty(z.shape[0], z.shape[1], dtype=z.dtype, device=z.device)
+    kernels().gelu(z, out)
+    return out
+
+
+def rot_kv_write(src: torch.Tensor, positions: torch.Tensor, slots: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor,
+                 H: int, G: int, scale: float, rot_dims: int = 0, freq: Optional[torch.Tensor] = None, mult: float = 1.0,
+                 vfreq: Optional[torch.Tensor] = None, wq: Optional[torch.Tensor] = None, wk: Optional[torch.Tensor] = None,
+                 eps: float = 0.0, q_out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """Cache side of a rotary attention layer.  ``src`` rows = [q (H D) | k (G D) | v (G Dv)].  With ``wq`` / ``wk`` (fp32
+    [D]) q / k are first RMS-normed per head (x / rms(x) * w).  The first ``rot_dims`` entries of every q and k head are
+    rotated by the position: entry i < rot_dims / 2 pairs with i + rot_dims / 2, angle position * freq[i], cos and sin
+    times ``mult``.  q times ``scale`` -> fp32 [T, H D] (returned); k -> the paged K cache at ``slots`` (-1: no write);
+    v -> the paged V cache, with ``vfreq`` (fp32 [Dv / 2]) rotated the same way over all its Dv entries."""
+    D = k_cache.shape[2] // G
+    if q_out is None:
+        q_out = torch.empty(src.shape[0], H * D, dtype=torch.float32, device=src.device)
+    kernels().rot_kv_write(src, wq, wk, freq, float(mult), int(rot_dims), vfreq, positions, slots, q_out, k_cache, v_cache,
+                           int(H), int(G), float(eps), float(scale))
+    return q_out
+
+
+def head_gate_unrotate(o: torch.Tensor, out: torch.Tensor, positions: torch.Tensor, H: int, gate: Optional[torch.Tensor] = None,
+                       vfreq: Optional[torch.Tensor] = None, scale: float = 1.0) -> torch.Tensor:
+    """out[t, h] = rot(o[t, h], -position) * sigmoid(gate[t, h]) * scale: the output of an attention over rotated values
+    turned back by the row's own position (``vfreq`` None: no rotation), one gate logit per head (``gate`` [T, H])."""
+    kernels().head_gate_unrotate(o, gate, vfreq, positions, out, int(H), float(scale))
+    return out
+
+
+def add_rmsnorm(x: torch.Tensor, y: Optional[torch.Tensor], w: torch.Tensor, eps: float, dtype,
+                out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """x (fp32) += y in place (``y`` None: x as it is), and x / rms(x) * w of the new x -> ``dtype`` rows."""
+    if out is None:
+        out = torch.empty(x.shape[0], x.shape[1], dtype=dtype, device=x.device)
+    kernels().add_rmsnorm(x, y, w, out, float(eps))
+    return out
+
+
+def channel_decay_rule(src: torch.Tensor, z: torch.Tensor, state: torch.Tensor, items: StepItems, H: int, G: int,
+                       zb: Optional[torch.Tensor] = None, A_log: Optional[torch.Tensor] = None, tau: float = 1.0,
+                       beta: Optional[torch.Tensor] = None, unit: bool = False, delta: bool = False,
+                       out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """Linear-attention recurrence with one decay per head and key channel over a step's items.  ``src`` rows
+    [q (G D) | k (G D) | v (H Dv)] (head h reads q / k head h // (H / G)); q times D^-1/2, with ``unit`` q and k first
+    made unit vectors per head.  Decays g [T, H D] from the logits ``z`` (+ ``zb``): with ``A_log`` (fp32 [H])
+    g = exp(-exp(A_log_h) softplus(z)), else g = sigmoid(z)^(1/tau).  Per head, g scaling the rows of S:
+    ``delta``: S <- g S; u = sigmoid(beta_h) (v - S^T k); S <- S + k u^T; else S <- g S + k v^T.  o = S^T q.
+    ``state`` fp32 [slots, H, D, Dv] (read unless the item starts at position 0, written back).  Returns o fp32
+    [T, H Dv]; an fp32 ``src`` is rewritten in place with the q and k that enter the recurrence."""
+    T = src.shape[0]
+    if out is None:
+        out = torch.empty(T, H * state.shape[3], dtype=torch.float32, device=src.device)
+    qkv = src if src.dtype == torch.float32 else torch.empty(T, src.shape[1], dtype=torch.float32, device=src.device)
+    kernels().chan_rule(src, qkv, z, zb, A_log, 1.0 / float(tau), beta, state, items.cu, items.slots, items.positions, out,
+                        int(H), int(G), bool(unit), bool(delta))
     return out
