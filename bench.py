@@ -57,8 +57,8 @@ def parse():
     ap.add_argument("--compare-layers", type=int, default=4, help="--compare-decoders: layers per model")
     ap.add_argument("--window", type=int, default=0, help="--compare-decoders: Madipel's window (0: the whole context)")
     ap.add_argument("--designs", default="madipel,llama",
-                    help="--compare-decoders: designs to run (madipel, llama, merudra, mixtral, limatar)")
-    ap.add_argument("--pattern", default="ad", help="--compare-decoders: mixer kinds per layer, repeated: a(ttention) / d(elta) for Merudra, l(ow-rank attention) / r(etention) for Limatar")
+                    help="--compare-decoders: designs to run (madipel, llama, merudra, mixtral, limatar, rerozen)")
+    ap.add_argument("--pattern", default="ad", help="--compare-decoders: mixer kinds per layer, repeated: a(ttention) / d(elta) for Merudra, l(ow-rank attention) / r(etention) for Limatar, p(arallel) / 2 (parallel_2) for Rerozen")
     return ap.parse_args()
 
 

@@ -3,12 +3,15 @@
 
     python bench.py --compare-decoders [--sizes small,8b-layer] [--compare-layers 4]
 
-Designs: ``madipel``, ``llama``, ``merudra``, ``mixtral``, ``limatar`` (``--designs merudra,mixtral`` puts Merudra
+Designs: ``madipel``, ``llama``, ``merudra``, ``mixtral``, ``limatar``, ``rerozen`` (``--designs merudra,mixtral`` puts Merudra
 beside the closest existing decoder, the routed-experts Mixtral: 8 experts, 2 per token, the same active feed-forward
 width; Merudra's layers alternate attention and gated delta rule mixers and add 2 identity experts.
 ``--designs limatar,merudra`` puts Limatar beside Merudra, the closest decoder with paged attention AND recurrent
 layers over an fp32 stream: Limatar's layers alternate low-rank attention (latent 512 + 64 rotated entries, sinks) and
 retention, routed experts with a shared expert and the clamped dense unit).
+``--designs rerozen,merudra`` puts Rerozen beside Merudra, the closest decoder (input convolutions in front of every
+sublayer, paged attention and gated delta rule layers over an fp32 stream): every Rerozen layer runs a chunked rotary
+attention AND a half-size channel-decay linear attention side by side, and a dense gelu feed-forward).
 
 For each size a Madipel model (parallel layers, windowed attention with distance bias, xIELU feed-forward, fp32
 residual) and the closest existing decoder (Llama: sequential layers, causal GQA attention with RoPE, SwiGLU) are
@@ -97,6 +100,33 @@ def _limatar(size: dict, layers: int, device, seed: int, experts: int = 8, top: 
     return LimatarModel(cfg, device=device, seed=seed)
 
 
+def _rerozen(size: dict, layers: int, device, seed: int, pattern: str = "p2", chunk: int = 1024):
+    """Layers alternating (``pattern``: p / 2 per layer, repeated; a / d and l / r of the other designs' patterns mean the
+    same) between "parallel" (attention with biases and q / k norms beside gated linear attention) and "parallel_2"
+    (attention with short convolutions, rotated values and a sink beside the gated delta rule).  The attention has the
+    other designs' heads and head size and chunks of ``chunk`` positions; the linear attention half as many heads of the
+    same size; the ungated feed-forward's two matrices get 1.5x the gated designs' inner width (equal parameters)."""
+    from llm_weighted_consensus_amd.models.config import RerozenConfig
+    from llm_weighted_consensus_amd.models.rerozen import RerozenModel
+
+    H, G, D, d = size["heads"], size["kv_heads"], size["head_dim"], size["width"]
+    rot = {"base": 10000.0, "dims": D // 2, "scaling": {"factor": 4.0, "original": 1024, "fast": 32.0, "slow": 1.0}}
+    left = {"heads": H, "kv_heads": G, "dim": D, "vdim": D, "scale": D ** -0.5, "mask": {"size": chunk}, "rot": rot}
+    mlp = {"kind": "dense", "ff": 3 * size["ffn"] // 2}
+    two = {"type": "parallel_2", "mlp": mlp,
+           "mixer": {"left": dict(left, conv=4), "right": {"heads": H // 2, "kv_heads": max(G // 2, 1), "dim": D, "vdim": D, "conv": 4,
+                                                           "a_rank": 64, "g_rank": 64},
+                     "left_scale": 0.7, "right_scale": 1.1}}
+    one = {"type": "parallel", "mlp": mlp,
+           "mixer": {"left": left, "right": {"heads": H // 2, "dim": D, "vdim": D, "tau": 16.0, "a_rank": 64},
+                     "left_scale": 1.2, "right_scale": 0.5}}
+    kinds = {"p": one, "a": one, "l": one, "2": two, "d": two, "r": two}
+    cfg = RerozenConfig.from_dict({"architecture": "Rerozen", "canon": {"taps": 4}, "embedding": {"scale": d ** 0.5},
+                                   "layers": [kinds[pattern[i % len(pattern)]] for i in range(layers)], "logit_scale": 0.25,
+                                   "norm": {"eps": 1e-6}, "vocab": size["vocab"], "width": d}, name="rerozen-bench")
+    return RerozenModel(cfg, device=device, seed=seed)
+
+
 def _mixtral(size: dict, layers: int, max_pos: int, device, seed: int, experts: int = 8, top: int = 2):
     from llm_weighted_consensus_amd.models.config import DecoderConfig
     from llm_weighted_consensus_amd.models.mixtral import MixtralModel
@@ -156,7 +186,9 @@ def run(sizes: str = "small,8b-layer", layers: int = 4, prompt_len: int = 2048, 
             if design == "madipel":
                 model = _madipel(size, layers, window, dev, 3)
             elif design == "merudra":
-                model = _merudra(size, layers, dev, 3, pattern="".join({"l": "a", "r": "d"}.get(c, c) for c in pattern))
+                model = _merudra(size, layers, dev, 3, pattern="".join({"l": "a", "r": "d", "p": "a", "2": "d"}.get(c, c) for c in pattern))
+            elif design == "rerozen":
+                model = _rerozen(size, layers, dev, 3, pattern=pattern)
             elif design == "limatar":
                 model = _limatar(size, layers, dev, 3, pattern=pattern)
             elif design == "mixtral":
@@ -172,7 +204,7 @@ def run(sizes: str = "small,8b-layer", layers: int = 4, prompt_len: int = 2048, 
                     **{k: round(v, 3) for k, v in r.items()}, "dtype": "bf16", "data": "synthetic"}
             print(json.dumps(line), flush=True)
             summary.setdefault(name, {})[design] = r
-    for a, b in (("madipel", "llama"), ("merudra", "mixtral"), ("merudra", "madipel"), ("limatar", "merudra")):
+    for a, b in (("madipel", "llama"), ("merudra", "mixtral"), ("merudra", "madipel"), ("limatar", "merudra"), ("rerozen", "merudra")):
         out = {}
         for name, d in summary.items():
             if a in d and b in d:

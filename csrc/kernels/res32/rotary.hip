@@ -94,6 +94,106 @@ __global__ void head_gate_unrotate_kernel(const AT* __restrict__ o, int ldi, con
   }
 }
 
+// cos / sin of one row's angles, shared by all heads: tab[m] = mult cos(pos f_m), tab[n + m] = mult sin(pos f_m)
+LWC_DEVICE void angle_table(float* tab, const float* freq, int n, float mult, float pos) {
+  for (int m = threadIdx.x; m < n; m += blockDim.x) {
+    float sn, cs;
+    sincosf(pos * freq[m], &sn, &cs);
+    tab[m] = cs * mult;
+    tab[n + m] = sn * mult;
+  }
+}
+
+// four consecutive entries [i, i + 4) of a head at src, rotated on the head's first rd entries with the table (rd / 2
+// a multiple of four), norm factors applied first (w may be null)
+template <typename IT>
+LWC_DEVICE float4v rotate4(const IT* src, int i, int rd, const float* tab, const float* w, float rstd) {
+  float4v x = Vec4<IT>::ld(src + i);
+  if (w) x *= Vec4<float>::ld(w + i) * rstd;
+  if (i < rd) {
+    const int half = rd >> 1;
+    const bool first = i < half;
+    const int m = first ? i : i - half, j = first ? i + half : i - half;
+    float4v xp = Vec4<IT>::ld(src + j);
+    if (w) xp *= Vec4<float>::ld(w + j) * rstd;
+    const float4v cs = Vec4<float>::ld(tab + m), sn = Vec4<float>::ld(tab + half + m);
+    x = first ? x * cs - xp * sn : x * cs + xp * sn;
+  }
+  return x;
+}
+
+// D, Dv multiples of four, rd and (rotated) Dv multiples of eight, every base a multiple of four entries: the angles
+// of a row are formed once for all heads, 8- / 16-byte accesses except the interleaved value stores.
+template <typename IT, typename CT>
+__global__ void __launch_bounds__(256) rot_kv_write_vec_kernel(
+    const IT* __restrict__ src, int lds, const float* __restrict__ wq, const float* __restrict__ wk,
+    const float* __restrict__ freq, float mult, int rd, const float* __restrict__ vfreq, const int* __restrict__ positions,
+    const int* __restrict__ slots, float* __restrict__ q_out, CT* __restrict__ k_cache, CT* __restrict__ v_cache,
+    long long kb_stride, long long vb_stride, int block_size, int H, int G, int D, int Dv, float eps, float scale) {
+  extern __shared__ __attribute__((aligned(16))) float sh[];  // [rd] angles of q / k | [Dv] angles of v | [H + G] norm factors
+  float* tab = sh;
+  float* vtab = sh + rd;
+  float* rstd_s = vtab + (vfreq ? Dv : 0);
+  const int t = blockIdx.x;
+  const int lane = threadIdx.x & 63, wv = threadIdx.x >> 6, nw = blockDim.x >> 6;
+  const IT* pr = src + (size_t)t * lds;
+  const float pos = (float)positions[t];
+  const int slot = slots[t];
+  const bool write = slot >= 0;
+  const long long blk = write ? slot / block_size : 0, off = write ? slot % block_size : 0;
+  const int nq = H * D, nk = G * D, nv = G * Dv;
+  if (rd) angle_table(tab, freq, rd >> 1, mult, pos);
+  if (vfreq) angle_table(vtab, vfreq, Dv >> 1, 1.0f, pos);
+  if (wq) {  // per-head norms: one wave per head
+    for (int h = wv; h < H + G; h += nw) {
+      const IT* x = pr + (size_t)h * D;  // the k heads follow the q heads
+      float s = 0.f;
+      for (int i = lane * 4; i < D; i += 256) {
+        const float4v v = Vec4<IT>::ld(x + i);
+        s += v[0] * v[0] + v[1] * v[1] + v[2] * v[2] + v[3] * v[3];
+      }
+      s = wave_sum(s);
+      if (lane == 0) rstd_s[h] = 1.0f / sqrtf(s / (float)D + eps);
+    }
+  }
+  __syncthreads();
+  const int d4 = D >> 2, dv4 = Dv >> 2;
+  const int uq = H * d4, uk = write ? G * d4 : 0, uv = write ? G * dv4 : 0;
+  for (int u = threadIdx.x; u < uq + uk + uv; u += blockDim.x) {
+    if (u < uq + uk) {
+      const int h = u / d4, i = (u - h * d4) * 4;  // h < H: a query head, else key head h - H
+      const float4v x = rotate4<IT>(pr + (size_t)h * D, i, rd, tab, h < H ? wq : wk, wq ? rstd_s[h] : 1.0f);
+      if (h < H) Vec4<float>::st(q_out + (size_t)t * nq + (size_t)h * D + i, x * scale);
+      else Vec4<CT>::st(k_cache + blk * kb_stride + off * nk + (size_t)(h - H) * D + i, x);
+    } else {
+      const int e = u - uq - uk, g = e / dv4, i = (e - g * dv4) * 4;
+      const float4v x = rotate4<IT>(pr + nq + nk + (size_t)g * Dv, i, vfreq ? Dv : 0, vtab, nullptr, 1.0f);
+      // V is 4-token interleaved: [block][offset / 4][column][offset % 4]
+      CT* vc = v_cache + blk * vb_stride + (off >> 2) * (4LL * nv) + (off & 3) + 4LL * (g * Dv + i);
+#pragma unroll
+      for (int c = 0; c < 4; ++c) Elem<CT>::st(vc + 4 * c, x[c]);
+    }
+  }
+}
+
+template <typename AT>
+__global__ void __launch_bounds__(256) head_gate_unrotate_vec_kernel(const AT* __restrict__ o, int ldi, const AT* __restrict__ g,
+                                                                      int ldg, const float* __restrict__ vfreq,
+                                                                      const int* __restrict__ positions, AT* __restrict__ out,
+                                                                      int ldo, int H, int Dv, float scale) {
+  extern __shared__ __attribute__((aligned(16))) float sh[];  // [Dv] angles
+  const int t = blockIdx.x;
+  if (vfreq) angle_table(sh, vfreq, Dv >> 1, 1.0f, -(float)positions[t]);  // turned back: the angles' signs flip
+  __syncthreads();
+  const int dv4 = Dv >> 2;
+  for (int u = threadIdx.x; u < H * dv4; u += blockDim.x) {
+    const int h = u / dv4, i = (u - h * dv4) * 4;
+    const float gate = scale * (g ? sigmoid_f(Elem<AT>::ld(g + (size_t)t * ldg + h)) : 1.0f);
+    const float4v x = rotate4<AT>(o + (size_t)t * ldi + (size_t)h * Dv, i, vfreq ? Dv : 0, sh, nullptr, 1.0f);
+    Vec4<AT>::st(out + (size_t)t * ldo + (size_t)h * Dv + i, x * gate);
+  }
+}
+
 template <typename YT, typename OT>
 __global__ void add_rmsnorm_kernel(float* __restrict__ x, const YT* __restrict__ y, int ldy, const float* __restrict__ w,
                                    OT* __restrict__ out, int ldo, int d, float eps) {
@@ -155,10 +255,20 @@ extern "C" int r32_rot_kv_write(const void* src, int lds, const float* wq, const
                                 int H, int G, int D, int Dv, float eps, float scale, int io, hipStream_t s) {
   if (T <= 0) return 0;
   if (rd < 0 || rd > D || (rd & 1) || (rd > 0 && !freq) || (vfreq && (Dv & 1))) return -1;
+  const int ib = (io & 1) ? 16 : 8, cb = (io & 2) ? 16 : 8;
+  const bool vec = D % 4 == 0 && Dv % 4 == 0 && rd % 8 == 0 && (!vfreq || Dv % 8 == 0) && lds % 4 == 0 && kb_stride % 4 == 0 &&
+                   (!wq == !wk) && aligned_to(src, ib) && aligned_to(k_cache, cb) && aligned_to(q_out, 16) &&
+                   aligned_to(wq, 16) && aligned_to(wk, 16);
+  const size_t shm = (size_t)(rd + (vfreq ? Dv : 0) + H + G) * sizeof(float);
 #define LWC_ROT(IT, CT)                                                                                                \
-  rot_kv_write_kernel<IT, CT><<<T, 256, 0, s>>>((const IT*)src, lds, wq, wk, freq, mult, rd, vfreq, positions, slots,   \
-                                                q_out, (CT*)k_cache, (CT*)v_cache, kb_stride, vb_stride, block_size, H, \
-                                                G, D, Dv, eps, scale)
+  if (vec)                                                                                                             \
+    rot_kv_write_vec_kernel<IT, CT><<<T, 256, shm, s>>>((const IT*)src, lds, wq, wk, freq, mult, rd, vfreq, positions, \
+                                                        slots, q_out, (CT*)k_cache, (CT*)v_cache, kb_stride, vb_stride, \
+                                                        block_size, H, G, D, Dv, eps, scale);                           \
+  else                                                                                                                 \
+    rot_kv_write_kernel<IT, CT><<<T, 256, 0, s>>>((const IT*)src, lds, wq, wk, freq, mult, rd, vfreq, positions, slots, \
+                                                  q_out, (CT*)k_cache, (CT*)v_cache, kb_stride, vb_stride, block_size,  \
+                                                  H, G, D, Dv, eps, scale)
   if (io == 3) {
     LWC_ROT(float, float);
   } else if (io == 0) {
@@ -179,6 +289,18 @@ extern "C" int r32_head_gate_unrotate(const void* o, int ldi, const void* g, int
   if (T <= 0) return 0;
   if (vfreq && (Dv & 1)) return -1;
   const int threads = H >= 4 ? 256 : 64 * H;
+  const int ab = f32 ? 16 : 8;
+  if (Dv % 4 == 0 && (!vfreq || Dv % 8 == 0) && ldi % 4 == 0 && ldo % 4 == 0 && aligned_to(o, ab) && aligned_to(out, ab)) {
+    const size_t shm = (size_t)(vfreq ? Dv : 4) * sizeof(float);
+    if (f32)
+      head_gate_unrotate_vec_kernel<float><<<T, 256, shm, s>>>((const float*)o, ldi, (const float*)g, ldg, vfreq, positions,
+                                                                (float*)out, ldo, H, Dv, scale);
+    else
+      head_gate_unrotate_vec_kernel<bf16_t><<<T, 256, shm, s>>>((const bf16_t*)o, ldi, (const bf16_t*)g, ldg, vfreq,
+                                                                 positions, (bf16_t*)out, ldo, H, Dv, scale);
+    LWC_CHECK_LAUNCH();
+    return 0;
+  }
   if (f32)
     head_gate_unrotate_kernel<float><<<T, threads, 0, s>>>((const float*)o, ldi, (const float*)g, ldg, vfreq, positions,
                                                             (float*)out, ldo, H, Dv, scale);

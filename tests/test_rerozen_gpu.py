@@ -279,6 +279,41 @@ def test_channel_decay_recurrences(gpu, dtype, H, G, D, Dv, delta):
         assert (state[slot[s]].cpu().double() - Sref[s]).abs().max() / Sref[s].abs().max().clamp_min(1.0) < tol, s
 
 
+@pytest.mark.parametrize("delta", [False, True])
+def test_channel_decay_many_sequences_at_once(gpu, delta):
+    """64 sequences side by side, two steps each (a grid large enough for the quarter-column split at D = 64): a portion
+    of three rows, then single rows, against the oracle."""
+    from llm_weighted_consensus_amd.ops import res32
+
+    g = torch.Generator().manual_seed(3)
+    B, H, G, D, Dv, n = 64, 8, 4, 64, 64, 5
+    src = torch.randn(B, n, 2 * G * D + H * Dv, generator=g)
+    z = torch.randn(B, n, H * D, generator=g) + 2.0
+    b = torch.randn(B, n, H, generator=g)
+    A_log = torch.rand(H, generator=g) - 2
+    state = (torch.randn(B + 1, H, D, Dv, generator=g) * 9).to(gpu)
+    slots = torch.randperm(B, generator=g).tolist()
+    got = torch.empty(B, n, H * Dv)
+    for a, c in ((0, 3), (3, 1), (4, 1)):
+        rows = lambda x: x[:, a:a + c].reshape(B * c, -1).contiguous().to(gpu)  # noqa: E731
+        o = res32.channel_decay_rule(rows(src), rows(z), state, _items([c] * B, slots, [a] * B, gpu), H, G,
+                                     A_log=A_log.to(gpu) if delta else None, tau=3.0, beta=rows(b) if delta else None,
+                                     unit=delta, delta=delta)
+        got[:, a:a + c] = o.cpu().view(B, c, H * Dv)
+    for s in (0, 17, 63):
+        q, k = src[s, :, :G * D].double().view(n, G, D), src[s, :, G * D:2 * G * D].double().view(n, G, D)
+        v = src[s, :, 2 * G * D:].double().view(n, H, Dv)
+        if delta:
+            q, k = q / torch.sqrt((q * q).sum(-1, keepdim=True) + 1e-6), k / torch.sqrt((k * k).sum(-1, keepdim=True) + 1e-6)
+            dec = torch.exp(-torch.exp(A_log.double())[None, :, None] * torch.nn.functional.softplus(z[s].double().view(n, H, D)))
+        else:
+            dec = (torch.sigmoid(z[s].double()) ** (1 / 3.0)).view(n, H, D)
+        ref, S = O.recurrence((q * D ** -0.5).repeat_interleave(H // G, 1), k.repeat_interleave(H // G, 1), v, dec,
+                              torch.sigmoid(b[s].double()) if delta else None)
+        assert (got[s].double().view(n, H, Dv) - ref).abs().max() / ref.abs().max().clamp_min(1.0) < 2e-4, s
+        assert (state[slots[s]].cpu().double() - S).abs().max() / S.abs().max().clamp_min(1.0) < 2e-4, s
+
+
 def test_far_token_survives_a_slow_decay(gpu):
     """A value written 400 tokens back under decays near one is read out with its exact weight: the product of the
     decays of its key channel since then (nothing else is written on that channel)."""
