@@ -53,13 +53,14 @@ __global__ void gelu_kernel(const AT* __restrict__ in, int ldi, AT* __restrict__
   }
 }
 
+// four columns per thread, rows along the grid's second dimension (no division per element)
 template <typename AT>
-__global__ void gelu_vec_kernel(const AT* __restrict__ in, int ldi, AT* __restrict__ out, int ldo, int n4, long long total4) {
-  for (long long e = (long long)blockIdx.x * blockDim.x + threadIdx.x; e < total4; e += (long long)gridDim.x * blockDim.x) {
-    const long long t = e / n4;
-    const int c = 4 * (int)(e - t * n4);
-    const float4v z = Vec4<AT>::ld(in + t * ldi + c);
-    Vec4<AT>::st(out + t * ldo + c, float4v{gelu_erf_f(z[0]), gelu_erf_f(z[1]), gelu_erf_f(z[2]), gelu_erf_f(z[3])});
+__global__ void gelu_vec_kernel(const AT* __restrict__ in, int ldi, AT* __restrict__ out, int ldo, int n4, int T) {
+  const int c = 4 * (blockIdx.x * blockDim.x + threadIdx.x);
+  if (c >= 4 * n4) return;
+  for (int t = blockIdx.y; t < T; t += gridDim.y) {
+    const float4v z = Vec4<AT>::ld(in + (size_t)t * ldi + c);
+    Vec4<AT>::st(out + (size_t)t * ldo + c, float4v{gelu_erf_f(z[0]), gelu_erf_f(z[1]), gelu_erf_f(z[2]), gelu_erf_f(z[3])});
   }
 }
 
@@ -109,8 +110,9 @@ extern "C" int r32_gelu(const void* in, int ldi, void* out, int ldo, int T, int 
   if (total <= 0) return 0;
   const int ab = f32 ? 16 : 8;
   const bool vec = n % 4 == 0 && ldi % 4 == 0 && ldo % 4 == 0 && aligned_to(in, ab) && aligned_to(out, ab);
-  if (vec && f32) gelu_vec_kernel<float><<<glu_grid(total / 4), 256, 0, s>>>((const float*)in, ldi, (float*)out, ldo, n / 4, total / 4);
-  else if (vec) gelu_vec_kernel<bf16_t><<<glu_grid(total / 4), 256, 0, s>>>((const bf16_t*)in, ldi, (bf16_t*)out, ldo, n / 4, total / 4);
+  const dim3 vgrid((n / 4 + 255) / 256, T < 32768 ? T : 32768);
+  if (vec && f32) gelu_vec_kernel<float><<<vgrid, 256, 0, s>>>((const float*)in, ldi, (float*)out, ldo, n / 4, T);
+  else if (vec) gelu_vec_kernel<bf16_t><<<vgrid, 256, 0, s>>>((const bf16_t*)in, ldi, (bf16_t*)out, ldo, n / 4, T);
   else if (f32) gelu_kernel<float><<<glu_grid(total), 256, 0, s>>>((const float*)in, ldi, (float*)out, ldo, n, total);
   else gelu_kernel<bf16_t><<<glu_grid(total), 256, 0, s>>>((const bf16_t*)in, ldi, (bf16_t*)out, ldo, n, total);
   LWC_CHECK_LAUNCH();
