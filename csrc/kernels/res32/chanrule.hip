@@ -15,7 +15,7 @@
 //   chan_rule   the recurrence: the work split of delta_rule (a workgroup of NW waves per (item, head, 16 NW value
 //               columns), a quarter state column per lane (an eighth, 8 NW columns, when the grid would leave SIMDs
 //               with fewer than two waves), a token's k, q and g staged once through LDS,
-//               double-buffered, loads two tokens ahead).  With Sg = g S (one multiply per state element):
+//               double-buffered, loads five tokens ahead in straight-line code).  With Sg = g S (one multiply per state element):
 //               S^T k and S^T q over Sg in one pass, o = Sg^T q + (k . q) u, S = Sg + k u^T.
 #include "elem.h"
 
@@ -123,7 +123,8 @@ __global__ void __launch_bounds__(256) chan_prep_vec_kernel(const ST* __restrict
 }
 
 // RG lanes share a state column (RG = 4: 16 columns per wave; RG = 8: 8 columns per wave, twice the waves for small grids)
-template <int DPL, int NW, int DELTA, int RG>
+// ONE: every item is a single row (a decode step): nothing is fetched ahead and nothing staged for a next token.
+template <int DPL, int NW, int DELTA, int RG, bool ONE>
 __global__ void __launch_bounds__(64 * NW) chan_rule_kernel(const float* __restrict__ qkv, int ldq,
                                                              const float* __restrict__ dec, const float* __restrict__ bq,
                                                              float* __restrict__ state, long long slot_stride,
@@ -178,12 +179,20 @@ __global__ void __launch_bounds__(64 * NW) chan_rule_kernel(const float* __restr
     if (RG == 8) x += __shfl_xor(x, 8, 64);
     return row_sum4(x);
   };
-  Stage A, B;
-  fetch(r0, A);
-  stash(0, A);
-  float v = A.v, beta = A.beta, qk = A.qk;
-  if (r0 + 1 < r1) fetch(r0 + 1, A);
-  if (r0 + 2 < r1) fetch(r0 + 2, B);
+  // Four register stages: a token's operands are fetched five tokens before its turn (a trip to memory takes about
+  // as long as two tokens' arithmetic).  Every fetch is unconditional, past the item's end it repeats the last row, so
+  // the loop body is straight-line code and the waits count exactly the loads still in flight.
+  Stage st0, st1, st2, st3;
+  const int rl = r1 - 1;
+  fetch(r0, st0);
+  stash(0, st0);
+  float v = st0.v, beta = st0.beta, qk = st0.qk;
+  if (!ONE) {
+    fetch(min(r0 + 1, rl), st0);
+    fetch(min(r0 + 2, rl), st1);
+    fetch(min(r0 + 3, rl), st2);
+    fetch(min(r0 + 4, rl), st3);
+  }
   __syncthreads();
   auto step = [&](int row, int cur, Stage& next) {
     const float4v* ks = reinterpret_cast<const float4v*>(&kqg_s[cur][0][r * QLD]);
@@ -208,17 +217,26 @@ __global__ void __launch_bounds__(64 * NW) chan_rule_kernel(const float* __restr
     if (live && r == 0) out[(size_t)row * ldo + h * Dv + col] = sq + qk * u;
 #pragma unroll
     for (int j = 0; j < DPL; ++j) S[j] += kk[j] * u;
-    if (row + 1 < r1) {
-      stash(cur ^ 1, next);
-      v = next.v, beta = next.beta, qk = next.qk;
-      if (row + 3 < r1) fetch(row + 3, next);
-    }
+    if (ONE) return;
+    stash(cur ^ 1, next);  // (behind the last token: a buffer nobody reads)
+    v = next.v, beta = next.beta, qk = next.qk;
+    fetch(min(row + 5, rl), next);
     __syncthreads();
   };
-  for (int row = r0; row < r1; row += 2) {
-    step(row, 0, A);
-    if (row + 1 < r1) step(row + 1, 1, B);
+  int row = r0;
+  if (ONE) {
+    step(row, 0, st0);
+    row = r1;
   }
+  for (; row + 4 <= r1; row += 4) {
+    step(row, 0, st0);
+    step(row + 1, 1, st1);
+    step(row + 2, 0, st2);
+    step(row + 3, 1, st3);
+  }
+  if (row < r1) step(row, 0, st0);
+  if (row + 1 < r1) step(row + 1, 1, st1);
+  if (row + 2 < r1) step(row + 2, 0, st2);
   if (live) {
 #pragma unroll
     for (int j = 0; j < DPL; ++j)
@@ -270,13 +288,20 @@ extern "C" int r32_chan_rule(const void* src, int lds, int src_f32, float* qkv, 
   const long long waves4 = (long long)H * items * ((Dv + 15) / 16);
   const bool fine = waves4 < 2048 && D > 32;
   const int tiles = fine ? (Dv + 7) / 8 : (Dv + 15) / 16;
-#define LWC_RULE(DPL, NW, RG)                                                                                       \
-  if (delta)                                                                                                        \
-    chan_rule_kernel<DPL, NW, 1, RG><<<dim3(H * ((tiles + NW - 1) / NW), items), 64 * NW, 0, s>>>(                  \
-        qkv, ldq, dec, bq, state, slot_stride, cu, item_slot, positions, out, ldo, H, G, D, Dv, (tiles + NW - 1) / NW); \
-  else                                                                                                              \
-    chan_rule_kernel<DPL, NW, 0, RG><<<dim3(H * ((tiles + NW - 1) / NW), items), 64 * NW, 0, s>>>(                  \
-        qkv, ldq, dec, bq, state, slot_stride, cu, item_slot, positions, out, ldo, H, G, D, Dv, (tiles + NW - 1) / NW)
+  const bool one = T == items;  // every item a single row
+#define LWC_RULE_K(DPL, NW, DL, RG, ONE)                                                                            \
+  chan_rule_kernel<DPL, NW, DL, RG, ONE><<<dim3(H * ((tiles + NW - 1) / NW), items), 64 * NW, 0, s>>>(              \
+      qkv, ldq, dec, bq, state, slot_stride, cu, item_slot, positions, out, ldo, H, G, D, Dv, (tiles + NW - 1) / NW)
+#define LWC_RULE(DPL, NW, RG)                 \
+  if (delta && one) {                         \
+    LWC_RULE_K(DPL, NW, 1, RG, true);         \
+  } else if (delta) {                         \
+    LWC_RULE_K(DPL, NW, 1, RG, false);        \
+  } else if (one) {                           \
+    LWC_RULE_K(DPL, NW, 0, RG, true);         \
+  } else {                                    \
+    LWC_RULE_K(DPL, NW, 0, RG, false);        \
+  }
 #define LWC_RULE_NW(DPL, RG)   \
   if (tiles >= 4) {            \
     LWC_RULE(DPL, 4, RG);      \
@@ -304,6 +329,7 @@ extern "C" int r32_chan_rule(const void* src, int lds, int src_f32, float* qkv, 
   }
 #undef LWC_RULE_NW
 #undef LWC_RULE
+#undef LWC_RULE_K
   LWC_CHECK_LAUNCH();
   return 0;
 }
