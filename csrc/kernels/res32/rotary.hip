@@ -144,7 +144,11 @@ __global__ void __launch_bounds__(256) rot_kv_write_vec_kernel(
   const int nq = H * D, nk = G * D, nv = G * Dv;
   if (rd) angle_table(tab, freq, rd >> 1, mult, pos);
   if (vfreq) angle_table(vtab, vfreq, Dv >> 1, 1.0f, pos);
-  if (wq) {  // per-head norms: one wave per head
+  // D / 4 a power of two up to 64: the D / 4 threads that share a head in the loop below are neighbours in one wave
+  // and sum its squares among themselves; else one wave per head beforehand
+  const int d4 = D >> 2, dv4 = Dv >> 2;
+  const bool among = wq && d4 <= 64 && (d4 & (d4 - 1)) == 0;
+  if (wq && !among) {
     for (int h = wv; h < H + G; h += nw) {
       const IT* x = pr + (size_t)h * D;  // the k heads follow the q heads
       float s = 0.f;
@@ -157,12 +161,20 @@ __global__ void __launch_bounds__(256) rot_kv_write_vec_kernel(
     }
   }
   __syncthreads();
-  const int d4 = D >> 2, dv4 = Dv >> 2;
   const int uq = H * d4, uk = write ? G * d4 : 0, uv = write ? G * dv4 : 0;
   for (int u = threadIdx.x; u < uq + uk + uv; u += blockDim.x) {
     if (u < uq + uk) {
       const int h = u / d4, i = (u - h * d4) * 4;  // h < H: a query head, else key head h - H
-      const float4v x = rotate4<IT>(pr + (size_t)h * D, i, rd, tab, h < H ? wq : wk, wq ? rstd_s[h] : 1.0f);
+      float rstd = 1.0f;
+      if (among) {
+        const float4v v = Vec4<IT>::ld(pr + (size_t)h * D + i);
+        float sq = v[0] * v[0] + v[1] * v[1] + v[2] * v[2] + v[3] * v[3];
+        for (int m = d4 >> 1; m > 0; m >>= 1) sq += __shfl_xor(sq, m, 64);
+        rstd = 1.0f / sqrtf(sq / (float)D + eps);
+      } else if (wq) {
+        rstd = rstd_s[h];
+      }
+      const float4v x = rotate4<IT>(pr + (size_t)h * D, i, rd, tab, h < H ? wq : wk, rstd);
       if (h < H) Vec4<float>::st(q_out + (size_t)t * nq + (size_t)h * D + i, x * scale);
       else Vec4<CT>::st(k_cache + blk * kb_stride + off * nk + (size_t)(h - H) * D + i, x);
     } else {
