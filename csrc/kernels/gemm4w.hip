@@ -16,7 +16,7 @@
 // Per K tile (BK = 64) and wave: 16 NT MFMAs (8 m x NT n tiles x 2 k-steps of 32), 2 (8 + NT)
 // ds_read_b128 fragment reads, 8 + NT LDS-DMA pieces of 1 KiB (the workgroup moves the A | W tile).  LDS
 // holds two K tiles.  Register fragments are double-buffered by k-step: X = k-step 0, Y = k-step 1.  The main
-// loop (G4_TILE_H, hipBLASLt's MT256x256x64 segment shape, disassembled): seg A = the Y reads of tile R, one
+// loop (G4_TILE_H, hipBLASLt's MT256x256x64 segment shape): seg A = the Y reads of tile R, one
 // per k-step-0 MFMA, lgkmcnt(0), barrier; seg B = the rest of k-step 0 and most of k-step 1, carrying tile
 // R+2's DMA pieces one per ~5 MFMAs at raised wave priority, counted vmcnt, barrier; seg C = the last
 // k-step-1 MFMAs with the X reads of tile R+1.  vmcnt never reaches 0 inside the loop except for the last
@@ -416,7 +416,7 @@ __global__ void __launch_bounds__(256, 1) gemm4w_kernel(Params p) {
     for (int k = 0; k < G::Reads; ++k) rd1(smem, offA0, offB0, xa, xb, k);
 
     constexpr int M1 = 8 * NT;  // MFMAs of one k-step
-    // VAR 32: the library kernel's segment shape (hipBLASLt's MT256x256x64 DTL loop, disassembled: the same
+    // VAR 32: the library kernel's segment shape (hipBLASLt's MT256x256x64 DTL loop: the same
     // 128 MFMA / 32 ds_read_b128 / 16 LDS-DMA per K tile, two barriers).  seg A: the Y reads of tile R back
     // to back, one per k-step-0 MFMA, then a few more MFMAs, lgkmcnt(0), barrier; seg B: the long middle —
     // the rest of k-step 0 and most of k-step 1 — carrying the tile R+2 DMA pieces one per ~5 MFMAs at raised
