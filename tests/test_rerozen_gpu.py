@@ -579,6 +579,38 @@ def test_generation_chunked_prefill_and_forks(gpu, tmp_path):
     assert eng.bm.num_free == eng.bm.num_blocks and eng.bm.num_free_state_slots == 8
 
 
+def test_server_worker_factory_and_seeded_sampling(gpu, tmp_path):
+    """The server's worker factory on a model folder of the design: prefix caching is off for it (a cached head brings
+    no recurrent state), the state pool is there.  Seeded top-k sampling through the engine's sampler: the same seed
+    gives the same tokens, and every drawn token is among the oracle's k best next tokens given the engine's own
+    tokens so far (up to near-ties at the k-th place)."""
+    from safetensors.torch import save_file
+
+    from llm_weighted_consensus_amd.engine.group import build_engine
+    from llm_weighted_consensus_amd.engine.sampling import SamplingParams
+
+    c = CONFIGS["mixed"]
+    cfg, ranks = O.make_config(c["width"], c["vocab"], c["layers"], taps=c["taps"])
+    W = O.make_weights(cfg, ranks, 5)
+    d = tmp_path / "served"
+    d.mkdir()
+    (d / "config.json").write_text(json.dumps(cfg))
+    save_file({k: v.contiguous() for k, v in W.items()}, str(d / "model.safetensors"))
+    eng = build_engine({"model_dir": str(d), "dtype": "float32", "max_batch": 4, "max_model_len": 128, "kv_fraction": 0.001}, 0)
+    assert eng.state is not None and not eng.prefix_caching and eng.bm.num_state_slots == 4
+    prompt = _tokens(20, cfg["vocab"], 8)
+    out = eng.generate([prompt], SamplingParams(temperature=0.0, max_tokens=12, ignore_eos=True))
+    _check_greedy(cfg, W, prompt, out[0][0])
+    sp = SamplingParams(temperature=1.5, top_k=5, max_tokens=24, ignore_eos=True, seed=7)
+    one, two = eng.generate([prompt], sp)[0][0], eng.generate([prompt], sp)[0][0]
+    assert one == two and len(one) == 24
+    lg = O.forward(cfg, W, prompt + one[:-1])[len(prompt) - 1:]
+    for t, tok in enumerate(one):
+        assert float(lg[t].topk(5).values[-1] - lg[t, tok]) < 0.04, t
+    assert any(int(lg[t].argmax()) != tok for t, tok in enumerate(one))  # some draws are not the best token
+    assert eng.bm.num_free == eng.bm.num_blocks and eng.bm.num_free_state_slots == 4
+
+
 def test_trace_replay_command_line(gpu, tmp_path):
     """bin/trace_run as a user runs it: JSON lines in, ``done <step>`` lines and <step>.f32 files out; two sequences
     interleaved (portions beside single tokens, one sitting a step out), pages and slots given back at ``end``."""
