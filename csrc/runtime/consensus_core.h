@@ -4,7 +4,7 @@
 //   * SelectPfx / SelectPfxTree     src/score/completions/client.rs:1342-1631
 //   * get_vote                      src/score/completions/client.rs:1661-1800
 //   * tally + confidence            src/score/completions/client.rs:384-455
-// Deliberate fixes of reference quirks (SURVEY.md §7.4):
+// Deliberate fixes of reference quirks:
 //   * descent walks the key's letters until it reaches the leaf-parent branch instead of trusting
 //     `depth()` of the first child (unequal subtree depths for N > m^3 panicked in the reference);
 //   * a logprob match whose top-logprobs hold no sibling letter falls back to the one-hot vote

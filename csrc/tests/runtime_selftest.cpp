@@ -1,4 +1,4 @@
-// Host-runtime self test built with -fsanitize=address,undefined (SURVEY.md §5: sanitizers on host code;
+// Host-runtime self test built with -fsanitize=address,undefined (sanitizers on host code;
 // GPU sanitizers are not available on this pool).  Exercises the paths the engine drives every step:
 // block allocation / fork / copy-on-write / free churn, the key tree for many choice counts, vote
 // extraction with and without logprobs, tally and error unification.  Exit code 0 = pass; ASan/UBSan

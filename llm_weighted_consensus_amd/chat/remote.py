@@ -5,7 +5,7 @@ Same semantics as the reference DefaultClient (src/chat/completions/client.rs:19
   * the request is forced to `stream: true` (adding `stream_options.include_usage` if the caller was
     unary);
   * attempts = [(base, model) for base] + [(base, m) for m in models for base] — fallback models use the
-    ctx-rewritten bases (the reference used the unrewritten list: SURVEY §7.4 fix);
+    ctx-rewritten bases (the reference used the unrewritten list; fixed here);
   * each attempt probes the FIRST chunk; on error/empty the next attempt runs; the whole list is
     retried with exponential backoff (100 ms initial, x1.5, ±50 % jitter, 1 s cap, 40 s budget) using a
     per-request clock;

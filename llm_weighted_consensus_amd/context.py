@@ -3,7 +3,7 @@
 The reference threads a generic ``CTX`` through every trait (``chat::completions::Client<CTX>``,
 ``CtxHandler::handle`` rewriting the API bases per request: src/chat/completions/client.rs:25-32, 56-79;
 the OSS binary passes ``()``: src/main.rs:152,175,197,220).  Here the context carries what a serving
-deployment needs per request (SURVEY §1 [NEW]):
+deployment needs per request (new beside the reference):
 
 * ``trace_id``  — ``traceparent`` / ``x-request-id`` header or a fresh id; tags the engine's spans and
   timers and is echoed back in the ``x-request-id`` response header;

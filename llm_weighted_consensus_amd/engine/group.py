@@ -1,6 +1,5 @@
-"""EngineGroup: one engine WORKER PROCESS per GPU behind one front end (SURVEY.md §7.1 "EngineGroup (1
-worker/GPU), candidate router"; §5 "worker heartbeat; on GPU/worker failure, drain and reschedule its
-sequences to surviving GPUs").
+"""EngineGroup: one engine WORKER PROCESS per GPU behind one front end (one worker per GPU, a
+candidate router; worker heartbeat; on GPU / worker failure, drain and reschedule its sequences to surviving GPUs).
 
 * Each worker is a spawned process that owns one GPU and one `LLMEngine` (built from a JSON-able model
   spec by ``worker_factory``), reads requests from its own queue and sends each engine step's token

@@ -1,6 +1,6 @@
 """Model architecture configs (public shapes, random-init or safetensors weights).
 
-Shapes come from the public model configs named in SURVEY.md §2.3 (not from the reference, which
+Shapes come from the public model configs (not from the reference, which
 runs no model): Llama-3-8B, Mixtral-8x7B, Mistral-7B/e5-mistral-7b and the bge-* BERT encoders.
 Small variants exist for tests.
 """

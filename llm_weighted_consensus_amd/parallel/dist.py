@@ -1,7 +1,7 @@
 """Process-group bring-up and the collectives the framework uses (RCCL over xGMI on MI355X).
 
 One process per GPU; `torch.distributed` backend "nccl" IS RCCL on ROCm.  On CPU (tests) the same
-code runs over gloo.  Collectives used by the serving/bench paths:
+code runs over gloo.  Collectives used by the serving/bench paths (C1-C5):
 
   C1 all_gather of candidate embeddings  [n_local, d] -> [world, n_local, d]
   C2 voter shares / votes                leader <-> follower TCP links, not collectives: a dead peer must

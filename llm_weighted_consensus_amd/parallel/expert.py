@@ -1,4 +1,4 @@
-"""Expert parallelism (EP) for the MoE decoder: token dispatch / combine over all-to-all.
+"""Expert parallelism (EP) for the MoE decoder: token dispatch / combine over all-to-all (collective C4).
 
 Layout: the E experts are split into W contiguous blocks of E/W (rank r owns experts [r*El, (r+1)*El)),
 each with its FULL FFN (no column split, unlike TP).  Attention is data-parallel: every rank runs its own

@@ -1,4 +1,4 @@
-"""Batched voter tally (SURVEY K10b) for concurrent score requests.
+"""Batched voter tally for concurrent score requests.
 
 The reference tallies each request on its own (src/score/completions/client.rs:384-455):
 ``cw = Vᵀ w``, ``confidence = cw / Σ cw``, voter agreement ``a_l = V_l · confidence``.  One request is

@@ -1,4 +1,4 @@
-"""Fault injection for the local engine (SURVEY.md §5 "Failure detection / recovery / fault injection").
+"""Fault injection for the local engine (failure detection, recovery, fault injection).
 
 ``LWC_FAULT`` is a comma-separated list of ``kind[:arg]``:
 

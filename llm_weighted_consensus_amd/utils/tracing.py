@@ -1,4 +1,4 @@
-"""Tracing and timing (SURVEY.md §5 "Tracing / profiling"; the reference has none).
+"""Tracing and timing (the reference has none).
 
 * ``span(name)`` — a context manager around an engine phase (schedule / prefill / decode.launch /
   decode.process / embed ...).  It always feeds a cheap in-process aggregator (count, total and max

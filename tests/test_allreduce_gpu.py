@@ -303,7 +303,7 @@ def _selftest_worker(rank, world, port, q):
 
 
 def test_ipc_collectives_self_test_catches_broken_mapping(gpu):
-    """the IPC collectives check themselves against the process group at start-up, and a
+    """The IPC collectives check themselves against the process group at start-up, and a
     broken peer mapping is caught (CommFailure on every rank) instead of decoding garbage."""
     ctx = mp.get_context("spawn")
     q = ctx.Queue()

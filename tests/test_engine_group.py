@@ -153,7 +153,7 @@ def _wait_live(g, n, timeout=120):
 
 
 def test_dead_worker_is_respawned_and_serves_again():
-    """Recovery (SURVEY §5, VERDICT r4 #5): a worker killed mid-load is replaced by a fresh child process;
+    """Recovery: a worker killed mid-load is replaced by a fresh child process;
     live_workers() returns to full size within a bounded time and the replacement takes later requests."""
     g = EngineGroup({"delay": 0.02}, devices=[0, 0], factory=FACTORY, heartbeat_timeout=60, respawn_backoff_s=0.2)
     try:

@@ -1,4 +1,4 @@
-"""End-to-end on the GPU (SURVEY §7.2 step 5, the minimum slice): the ASGI server with a local
+"""End-to-end on the GPU (the minimum slice): the ASGI server with a local
 random-init Llama voter model and a local BGE encoder.  /score/completions with N voters that all map
 to the local engine (json_schema output mode: constrained decoding guarantees a parseable key; votes
 from real top-k logprobs), /chat/completions streaming, /multichat, /consensus, /embeddings — and

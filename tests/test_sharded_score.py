@@ -4,7 +4,7 @@ follower its share of voters over the shard links, merges their chunks live and 
 * world 2: a request's voters split across ranks give the single-process tally, confidences, votes and
   usage; "every vote failed" is decided over all voters (codes unified); concurrent requests; streamed
   requests interleave the follower's voter chunks live (before the final chunk);
-* world 4, failure isolation (VERDICT r3 item 2): a follower killed mid-load turns exactly its unfinished
+* world 4, failure isolation: a follower killed mid-load turns exactly its unfinished
   voters of the in-flight requests into ``voter_shard_lost`` error choices, those requests complete within
   the bound, later requests run on the survivors with every voter ok, and nothing waits for a process-group
   timeout;
@@ -360,7 +360,7 @@ def test_release_drops_a_share_whose_stream_never_ran():
 
 @pytest.mark.timeout(300)
 def test_restarted_follower_rejoins_and_serves(tmp_path):
-    """Recovery (VERDICT r4 #5): a follower dies mid-load (its voters become error choices), a restarted
+    """Recovery: a follower dies mid-load (its voters become error choices), a restarted
     process re-joins the running leader through the join file, live() returns to full size and later
     requests run voters on it again."""
     ctx = mp.get_context("spawn")

@@ -1,4 +1,4 @@
-"""Training-table voter weights that LEARN (SURVEY §2 row 23; reference types src/score/model/mod.rs:278-306,
+"""Training-table voter weights that LEARN (reference types src/score/model/mod.rs:278-306,
 stub src/score/completions/weight.rs:99-117): every scored request of a training-table model records
 the transcript embedding and each voter's agreement with the consensus; later requests with similar
 transcripts weight voters by that history; the table persists as JSONL and is replayed on start."""
